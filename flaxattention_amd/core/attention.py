@@ -1,0 +1,321 @@
+"""Front-ends: flax_attention, flax_attention_pallas, math_attention.
+
+Same names, arguments, defaults and errors as flaxattention/core/attention.py
+(flax_attention 169-218, flax_attention_pallas 220-312, math_attention 67-106,
+validators 119-167).  Arrays are torch tensors resident on the MI355X; the
+work is done by the HIP kernels behind include/flexattn.h, reached through
+ctypes.  Differentiation goes through a torch.autograd.Function that plays the
+role of the reference's jax.custom_vjp (kernel/attention.py:166-168, 653):
+forward saves (q, k, v, out, lse2), backward returns (dq, dk, dv).
+
+``kernel_options`` (accepted and ignored by the reference, attention.py:179)
+selects numerics here:
+    {"strict": True}    faithful kernels: S, normalised P, dP and dS are
+                        rounded through the input dtype exactly where the
+                        reference's dense path rounds them
+    {"round_s": bool}   fused kernels: round Q.K^T through the input dtype
+                        (default True, as attention.py:27 computes that product
+                        in the input dtype)
+    {"backend": "generic" | "auto"}
+    {"decode_splits": n}  force the split-KV decode kernel with n splits
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Callable, Dict, Optional, Tuple, Union
+
+import torch
+
+from .. import _lib
+from .blockmask import BlockMask, _create_empty_block_mask
+from .common import (IDENTITY, MaskMod, ScoreMod, _identity, _mask_mod_signature, _score_mod_signature,
+                     resolve_mask_mod, resolve_score_mod)
+
+Array = torch.Tensor
+
+_DTYPES = {torch.float32: _lib.FLEX_F32, torch.float16: _lib.FLEX_F16, torch.bfloat16: _lib.FLEX_BF16}
+
+
+def _validate_sdpa_input(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None):
+    """attention.py:119-138."""
+    if query.dtype != key.dtype or query.dtype != value.dtype:
+        raise ValueError(
+            f"Expected query, key, and value to have the same dtype, "
+            f"but got query.dtype: {query.dtype}, key.dtype: {key.dtype}, "
+            f"and value.dtype: {value.dtype} instead."
+        )
+    if query.dim() < 2 or key.dim() < 2 or value.dim() < 2:
+        raise ValueError(
+            f"Expected query, key, and value to all be  at least 2 dimensional, but got query.dim: "
+            f"{query.dim()}, key.dim: {key.dim()} and value.dim: {value.dim()} instead."
+        )
+
+
+def _validate_embed_dim(query, key, value):
+    """attention.py:149-167."""
+    if query.shape[-1] != key.shape[-1]:
+        raise ValueError(
+            f"Expect query and key/value to have the same embedding dimension "
+            f"but got E={query.shape[-1]} and E={key.shape[-1]}."
+        )
+    if value.shape[-1] > query.shape[-1]:
+        raise ValueError(
+            f"NYI: Currently value embedding dimension must be less than or equal to query embedding dimension. "
+            f"Got Ev={value.shape[-1]} and E={query.shape[-1]}."
+        )
+
+
+def _require_device(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise _lib.FlexAttnError("flaxattention_amd computes on the HIP device only: got a CPU tensor "
+                                     "(there is no CPU fallback)")
+    if ts[0].dtype not in _DTYPES:
+        raise TypeError(f"unsupported dtype {ts[0].dtype}; use float32, float16 or bfloat16")
+
+
+class _Plan:
+    """Everything but the tensors: the POD the C ABI takes plus what keeps its
+    device pointers alive."""
+
+    def __init__(self, q, k, v, score: ScoreMod, mask: MaskMod, block_mask: Optional[BlockMask], scale: float,
+                 flags: int, bhld: bool, decode_splits: int = 0):
+        # logical [B,H,L,D] views; physical layout may be [B,L,H,D]
+        self.B, self.Hq, self.Lq, self.D = q.shape
+        self.Hkv, self.Lkv, self.Dv = k.shape[1], k.shape[2], v.shape[3]
+        self.dtype = q.dtype
+        self.score, self.mask, self.block_mask = score, mask, block_mask
+        self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
+        self.lists = None
+        self.keep = [mask.bits]
+
+    def params(self, q, k, v, o) -> _lib.FlexAttnParams:
+        p = _lib.FlexAttnParams()
+        p.dtype = _DTYPES[self.dtype]
+        p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = self.B, self.Hq, self.Hkv, self.Lq, self.Lkv, self.D, self.Dv
+        for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
+            if t.stride(3) != 1:
+                raise _lib.FlexAttnError("the feature axis must be contiguous")
+            getattr(p, name)[:] = [t.stride(0), t.stride(1), t.stride(2)]
+        p.scale, p.flags = self.scale, self.flags
+        p.score = self.score.c_struct()
+        p.mask = self.mask.c_struct()
+        L = self.lists
+        if L is not None:
+            t = p.tiles
+            t.kv_num, t.kv_idx = L["kv_num_blocks"].data_ptr(), L["kv_indices"].data_ptr()
+            t.full_kv_num, t.full_kv_idx = L["full_kv_num_blocks"].data_ptr(), L["full_kv_indices"].data_ptr()
+            t.q_num, t.q_idx = L["q_num_blocks"].data_ptr(), L["q_indices"].data_ptr()
+            t.full_q_num, t.full_q_idx = L["full_q_num_blocks"].data_ptr(), L["full_q_indices"].data_ptr()
+            t.q_block, t.kv_block = L["q_block"], L["kv_block"]
+            t.n_q_blocks, t.n_kv_blocks = L["n_q_blocks"], L["n_kv_blocks"]
+            t.stride_b = 0 if L["B"] == 1 else L["H"]
+            t.stride_h = 0 if L["H"] == 1 else 1
+        return p
+
+
+def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, scale, kernel_options) -> _Plan:
+    opts = dict(kernel_options or {})
+    B, Hq, Lq, D = q.shape
+    Lkv = k.shape[2]
+    dev = q.device
+    score = resolve_score_mod(score_mod, Hq)
+    if block_mask is not None:
+        if block_mask.seq_lengths is not None and (block_mask.seq_lengths[0] < Lq or block_mask.seq_lengths[1] < Lkv):
+            raise ValueError(f"block_mask was built for lengths {block_mask.seq_lengths}, "
+                             f"but the inputs have Lq={Lq}, Lkv={Lkv}")
+        mask = block_mask.resolved_spec(B, Hq, Lq, Lkv, dev)
+    else:
+        mask = resolve_mask_mod(mask_mod, B, Hq, Lq, Lkv, dev)
+    flags = 0
+    if opts.get("strict", False):
+        flags |= _lib.FLAG_STRICT
+    if opts.get("round_s", True) and q.dtype != torch.float32:
+        flags |= _lib.FLAG_ROUND_S
+    if opts.get("backend", "auto") == "generic":
+        flags |= _lib.FLAG_FORCE_GENERIC
+    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, opts.get("decode_splits", 0))
+    # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
+    if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
+        qb, kvb = _lib.C.c_int32(0), _lib.C.c_int32(0)
+        _lib.lib().flexattn_preferred_tiles(_DTYPES[q.dtype], D, v.shape[3], Lq, Lkv, _lib.C.byref(qb), _lib.C.byref(kvb))
+        if qb.value > 0:
+            holder = block_mask if block_mask is not None else _holder_for(mask)
+            holder.spec = mask
+            plan.lists = holder.tile_lists(qb.value, kvb.value, B, Hq, Lq, Lkv, dev)
+    return plan
+
+
+_holders: dict = {}
+
+
+def _holder_for(mask: MaskMod) -> BlockMask:
+    """A cache object for tile lists of a mask that came without a BlockMask
+    (flax_attention_pallas takes a bare mask_mod)."""
+    key = mask.key()
+    h = _holders.get(key)
+    if h is None:
+        if len(_holders) > 64:
+            _holders.clear()
+        dev = mask.bits.device if mask.bits is not None else torch.device("cuda", torch.cuda.current_device())
+        h = BlockMask.from_kv_blocks(torch.ones([1, 1, 1], dtype=torch.int32, device=dev),
+                                     torch.zeros([1, 1, 1, 1], dtype=torch.int32, device=dev), mask_mod=mask)
+        _holders[key] = h
+    return h
+
+
+def _stream(t) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
+    L = _lib.lib()
+    o = torch.empty((plan.B, plan.Hq, plan.Lq, plan.Dv), dtype=q.dtype, device=q.device)
+    lse2 = torch.empty((plan.B, plan.Hq, plan.Lq), dtype=torch.float32, device=q.device)
+    p = plan.params(q, k, v, o)
+    with torch.cuda.device(q.device):
+        if plan.decode_splits > 0:
+            nbytes = L.flexattn_decode_workspace_bytes(p, plan.decode_splits)
+            ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+            rc = L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(),
+                                   plan.decode_splits, ws.data_ptr(), _stream(q))
+            _lib.check(rc, "flexattn_decode")
+        else:
+            rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), None, _stream(q))
+            _lib.check(rc, "flexattn_fwd")
+    return o, lse2
+
+
+def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o) -> Tuple[Array, Array, Array]:
+    L = _lib.lib()
+    d_o = d_o.contiguous()
+    dq = torch.empty((plan.B, plan.Hq, plan.Lq, plan.D), dtype=q.dtype, device=q.device)
+    dk = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.D), dtype=q.dtype, device=q.device)
+    dv = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.Dv), dtype=q.dtype, device=q.device)
+    p = plan.params(q, k, v, o)
+    with torch.cuda.device(q.device):
+        ws = torch.empty(max(L.flexattn_bwd_workspace_bytes(p), 256), dtype=torch.uint8, device=q.device)
+        rc = L.flexattn_bwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), d_o.data_ptr(),
+                            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), _stream(q))
+    _lib.check(rc, "flexattn_bwd")
+    return dq, dk, dv
+
+
+class _FlexAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, plan: _Plan):
+        o, lse2 = _run_fwd(plan, q, k, v)
+        ctx.save_for_backward(q, k, v, o, lse2)
+        ctx.plan = plan
+        ctx.mark_non_differentiable(lse2)
+        return o, lse2
+
+    @staticmethod
+    def backward(ctx, d_o, _d_lse):
+        q, k, v, o, lse2 = ctx.saved_tensors
+        dq, dk, dv = _run_bwd(ctx.plan, q, k, v, o, lse2, d_o)
+        return dq, dk, dv, None
+
+
+def _as_kernel_layout(t: Array) -> Array:
+    return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def math_attention(query: Array, key: Array, value: Array, score_mod: Callable, block_mask: Tuple, scale: float,
+                   kernel_options: Dict[str, Any], score_mod_other_buffers: Tuple = (),
+                   mask_mod_other_buffers: Tuple = (), use_pallas: bool = False) -> Tuple[Array, Array]:
+    """attention.py:67-106: (output, base-2 logsumexp).  ``block_mask`` is the
+    tuple BlockMask.as_tuple() gives; only its last entry (the mask_mod) is
+    read, as in the reference (attention.py:45).  Runs the faithful kernels."""
+    if score_mod_other_buffers or mask_mod_other_buffers:
+        raise NotImplementedError("captured buffers are not supported")
+    _require_device(query, key, value)
+    q, k, v = map(_as_kernel_layout, (query, key, value))
+    opts = dict(kernel_options or {})
+    opts.setdefault("strict", True)
+    plan = _make_plan(q, k, v, score_mod, None, block_mask[-1], scale, opts)
+    return _FlexAttention.apply(q, k, v, plan)
+
+
+def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_score_mod_signature] = None,
+                   block_mask: Optional[BlockMask] = None, scale: Optional[float] = None, enable_gqa: bool = False,
+                   return_lse: bool = False, kernel_options: Optional[Dict[str, Any]] = None
+                   ) -> Union[Array, Tuple[Array, Array]]:
+    """attention.py:169-218."""
+    _validate_sdpa_input(query, key, value)
+    _validate_embed_dim(query, key, value)
+    if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+        raise NotImplementedError("NYI: query, key, and value must be 4D tensors")
+    if (not enable_gqa) and query.shape[-3] != key.shape[-3]:
+        raise ValueError(
+            f"Expect query and key/value to have the same number of heads "
+            f"but got Hq={query.shape[-3]} and Hkv={key.shape[-3]}. "
+            f"Try setting enable_gqa=True for GQA."
+        )
+    if enable_gqa:
+        Hq = query.shape[1]
+        Hkv = key.shape[1]
+        if Hq % Hkv != 0:
+            raise ValueError(
+                f"Expect number of query heads to be a multiple of kv heads for GQA "
+                f"but got Hq={Hq} and Hkv={Hkv}."
+            )
+    _require_device(query, key, value)
+    if score_mod is None:
+        score_mod = _identity
+    if block_mask is None:
+        block_mask = _create_empty_block_mask(query, key)
+    if scale is None:
+        scale = 1.0 / math.sqrt(query.shape[-1])
+    q, k, v = map(_as_kernel_layout, (query, key, value))
+    plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
+    out, lse2 = _FlexAttention.apply(q, k, v, plan)
+    if return_lse:
+        return out, lse2 * math.log(2.0)
+    return out
+
+
+def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Optional[_score_mod_signature] = None,
+                          mask_mod: Optional[_mask_mod_signature] = None, block_q: int = 64, block_k: int = 64,
+                          sm_scale: Optional[float] = None, bhln: bool = True, enable_gqa: bool = False,
+                          block_mask: Optional[BlockMask] = None, block_mod: Optional[_mask_mod_signature] = None,
+                          kernel_options: Optional[Dict[str, Any]] = None) -> Array:
+    """attention.py:220-312: the fused-kernel front-end.  ``bhln=True`` takes
+    [B,H,L,D]; ``bhln=False`` takes [B,L,H,D] (read in place through strides).
+    ``block_q`` / ``block_k`` are accepted for compatibility; tile shapes are
+    chosen by the kernels.  ``block_mask=`` (a BlockMask) and the README's
+    spelling ``block_mod=`` are accepted next to ``mask_mod=``.  Unlike the
+    reference kernel (kernel/attention.py:233-235 indexes K/V with the q-head
+    id) GQA works here."""
+    if block_mod is not None:
+        if mask_mod is not None:
+            raise ValueError("pass only one of mask_mod= and block_mod=")
+        mask_mod = block_mod
+    if not bhln:
+        query, key, value = (t.transpose(1, 2) for t in (query, key, value))
+    _validate_sdpa_input(query, key, value)
+    _validate_embed_dim(query, key, value)
+    if query.dim() != 4 or key.dim() != 4 or value.dim() != 4:
+        raise NotImplementedError("NYI: query, key, and value must be 4D tensors")
+    if (not enable_gqa) and query.shape[1] != key.shape[1]:
+        raise ValueError(
+            f"Expect query and key/value to have the same number of heads "
+            f"but got Hq={query.shape[1]} and Hkv={key.shape[1]}. "
+            f"Try setting enable_gqa=True for GQA."
+        )
+    if enable_gqa:
+        Hq, Hkv = query.shape[1], key.shape[1]
+        if Hq % Hkv != 0:
+            raise ValueError(
+                f"Expect number of query heads to be a multiple of kv heads for GQA "
+                f"but got Hq={Hq} and Hkv={Hkv}."
+            )
+    _require_device(query, key, value)
+    if sm_scale is None:
+        sm_scale = 1 / math.sqrt(query.shape[-1])
+    if block_mask is not None and mask_mod is not None:
+        raise ValueError("pass only one of block_mask= and mask_mod=")
+    q, k, v = map(_as_kernel_layout, (query, key, value))
+    plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
+    out, _ = _FlexAttention.apply(q, k, v, plan)
+    return out if bhln else out.transpose(1, 2)

@@ -1,0 +1,367 @@
+"""Mod plumbing: signatures, arity-based classification and the functor objects
+that the HIP kernels understand.
+
+Mirrors flaxattention/core/common.py:7-39 (type aliases, _ModificationType,
+_get_mod_type).  The reference maps a *scalar* Python function over
+(b, h, q_idx, kv_idx) with four nested vmaps (common.py:41-80); here a mod is
+lowered to a small POD functor (FlexScoreMod / FlexMask in include/flexattn.h)
+that is evaluated inside the kernels.  The functor objects below are also plain
+callables with the reference's scalar signature, so user code that calls or
+combines them keeps working; they broadcast over torch tensors, numpy arrays
+and Python ints alike.
+"""
+from __future__ import annotations
+
+import inspect
+import math
+from enum import Enum
+from typing import Any, Callable, Optional
+
+import torch
+
+from .. import _lib
+
+Array = torch.Tensor
+_score_mod_signature = Callable[[Array, Array, Array, Array, Array], Array]
+_mask_mod_signature = Callable[[Array, Array, Array, Array], Array]
+
+INT_MIN, INT_MAX = _lib.INT_MIN, _lib.INT_MAX
+
+
+class _ModificationType(Enum):
+    """common.py:10-19."""
+    SCORE_MOD = 1
+    MASK_MOD = 2
+    UNKNOWN = 3
+
+
+def _get_mod_type(fn: Callable) -> _ModificationType:
+    """common.py:21-39: five positional arguments -> score_mod, four -> mask_mod."""
+    if isinstance(fn, ScoreMod):
+        return _ModificationType.SCORE_MOD
+    if isinstance(fn, MaskMod):
+        return _ModificationType.MASK_MOD
+    num_positional_args = sum(
+        1 for param in inspect.signature(fn).parameters.values()
+        if param.default == inspect.Parameter.empty
+    )
+    assert num_positional_args == 5 or num_positional_args == 4
+    if num_positional_args == 5:
+        return _ModificationType.SCORE_MOD
+    elif num_positional_args == 4:
+        return _ModificationType.MASK_MOD
+    return _ModificationType.UNKNOWN
+
+
+# ---------------------------------------------------------------------------
+# score_mod functors
+# ---------------------------------------------------------------------------
+def _f32(x):
+    if torch.is_tensor(x):
+        return x.to(torch.float32)
+    return x
+
+
+class ScoreMod:
+    """A score_mod the fused kernels evaluate in registers.
+
+    kind/p0/p1/i0 are the fields of FlexScoreMod.  Calling the object applies
+    the same scalar function to its arguments."""
+
+    def __init__(self, kind: int, p0: float = 0.0, p1: float = 0.0, i0: int = 0, name: str = "score_mod"):
+        self.kind, self.p0, self.p1, self.i0 = int(kind), float(p0), float(p1), int(i0)
+        self.__name__ = name
+
+    def c_struct(self) -> _lib.FlexScoreMod:
+        return _lib.FlexScoreMod(self.kind, self.p0, self.p1, self.i0, 0)
+
+    def key(self):
+        return (self.kind, self.p0, self.p1, self.i0)
+
+    def __call__(self, score, b, h, q_idx, kv_idx):
+        k = self.kind
+        if k == _lib.SCORE_IDENTITY:
+            return score
+        if k == _lib.SCORE_CHECKERBOARD:
+            par = ((kv_idx - q_idx) if self.i0 == 0 else (kv_idx + 0 * q_idx)) % 2
+            if torch.is_tensor(par):
+                return torch.where(par == 0, score * self.p0, score * self.p1)
+            return score * (self.p0 if par == 0 else self.p1)
+        if k == _lib.SCORE_ALIBI:
+            slope = 2.0 ** (-((_f32(h) + 1) * 8.0 / self.i0))
+            return score + _f32(q_idx - kv_idx) * slope * self.p0
+        if k == _lib.SCORE_TANH_SOFTCAP:
+            if torch.is_tensor(score):
+                return self.p0 * torch.tanh(score / self.p0)
+            return self.p0 * math.tanh(score / self.p0)
+        if k == _lib.SCORE_REL_BIAS:
+            return score + _f32(kv_idx - q_idx) * self.p0
+        raise ValueError(f"unknown score_mod kind {k}")
+
+    def __repr__(self):
+        return f"ScoreMod({self.__name__}, kind={self.kind}, p0={self.p0}, p1={self.p1}, i0={self.i0})"
+
+
+def _identity(score, batch, head, token_q, token_kv):
+    """flaxattention/core/attention.py:109-116."""
+    return score
+
+
+IDENTITY = ScoreMod(_lib.SCORE_IDENTITY, name="identity")
+
+
+def _probe_score_mod(fn: Callable, H: int) -> Optional[ScoreMod]:
+    """Recognise an untagged Python score_mod as one of the functor families by
+    evaluating it on a small CPU grid and checking every family exactly."""
+    P = 7
+    Hn = max(int(H), 1)
+    s = torch.tensor([-1.75, -0.5, 0.0, 0.625, 2.5], dtype=torch.float32).reshape(5, 1, 1, 1, 1)
+    b = torch.arange(2, dtype=torch.int32).reshape(1, 2, 1, 1, 1)
+    h = torch.arange(Hn, dtype=torch.int32).reshape(1, 1, Hn, 1, 1)
+    q = torch.arange(P, dtype=torch.int32).reshape(1, 1, 1, P, 1)
+    kv = torch.arange(P + 2, dtype=torch.int32).reshape(1, 1, 1, 1, P + 2)
+    shape = (5, 2, Hn, P, P + 2)
+    try:
+        out = fn(s.expand(shape), b, h, q, kv)
+        if not torch.is_tensor(out):
+            return None
+        out = torch.broadcast_to(out.to(torch.float32), shape)
+    except Exception:
+        return None
+
+    def same(c: ScoreMod) -> bool:
+        ref = torch.broadcast_to(_f32(c(s.expand(shape), b, h, q, kv)), shape)
+        return bool(torch.allclose(out, ref, rtol=1e-6, atol=1e-6))
+
+    cands = [IDENTITY]
+    # multiplicative checkerboards: read both factors off two grid points
+    with torch.no_grad():
+        one = out[4] / 2.5  # score 2.5
+        for i0 in (0, 1):
+            f_even = one[0, 0, 0, 0].item()
+            f_odd = one[0, 0, 0, 1].item()
+            cands.append(ScoreMod(_lib.SCORE_CHECKERBOARD, f_even, f_odd, i0, name=getattr(fn, "__name__", "checkerboard")))
+        bias = out[2]  # score 0
+        for sign in (1.0, -1.0):
+            cands.append(ScoreMod(_lib.SCORE_ALIBI, sign, 0.0, Hn, name=getattr(fn, "__name__", "alibi")))
+        cands.append(ScoreMod(_lib.SCORE_REL_BIAS, bias[0, 0, 0, 1].item(), name=getattr(fn, "__name__", "rel_bias")))
+        # tanh soft-cap: cap from the saturated value
+        try:
+            big = fn(torch.full((1, 1, 1, 1, 1), 1e9), b[:, :1], h[:, :, :1], q[..., :1, :], kv[..., :1])
+            cap = float(torch.as_tensor(big).reshape(-1)[0])
+            if math.isfinite(cap) and cap > 0:
+                cands.append(ScoreMod(_lib.SCORE_TANH_SOFTCAP, cap, 1.0 / cap, name=getattr(fn, "__name__", "tanh_softcap")))
+        except Exception:
+            pass
+    for c in cands:
+        if same(c):
+            return c
+    return None
+
+
+_score_cache: dict = {}
+
+
+def resolve_score_mod(fn: Optional[Callable], H: int) -> ScoreMod:
+    """Lower a score_mod callable to a kernel functor, or raise."""
+    if fn is None or fn is _identity:
+        return IDENTITY
+    if isinstance(fn, ScoreMod):
+        return fn
+    key = (id(fn), H)
+    hit = _score_cache.get(key)
+    if hit is not None and hit[0] is fn:
+        return hit[1]
+    spec = _probe_score_mod(fn, H)
+    if spec is None:
+        raise NotImplementedError(
+            "score_mod is not one of the fused functor families (identity, checkerboard, ALiBi, "
+            "tanh soft-cap, relative-position bias); build it with flaxattention_amd.mods.* "
+            "so the kernels can fuse it")
+    _score_cache[key] = (fn, spec)
+    return spec
+
+
+# ---------------------------------------------------------------------------
+# mask_mod functors
+# ---------------------------------------------------------------------------
+class MaskMod:
+    """A mask_mod the kernels evaluate: either the canonical band form
+
+        d = q_idx + q_offset - kv_idx
+        visible = (d >= lo) and (d <= hi or kv_idx <= sink)
+
+    or a packed bitmap made from an arbitrary callable (kind BITS)."""
+
+    def __init__(self, lo: int = INT_MIN, hi: int = INT_MAX, sink: int = -1, q_offset: int = 0,
+                 name: str = "mask_mod", bits: Optional[torch.Tensor] = None, fn: Optional[Callable] = None):
+        self.lo, self.hi, self.sink, self.q_offset = int(lo), int(hi), int(sink), int(q_offset)
+        self.bits = bits      # int32 [Bm, Hm, Qp, KVw] on the device, or None
+        self.fn = fn          # the callable a bitmap was made from
+        self.__name__ = name
+
+    @property
+    def kind(self) -> int:
+        return _lib.MASK_BITS if self.bits is not None else _lib.MASK_BAND
+
+    def is_noop(self) -> bool:
+        return self.bits is None and self.lo == INT_MIN and self.hi == INT_MAX
+
+    def key(self):
+        if self.bits is not None:
+            return ("bits", self.bits.data_ptr())
+        return ("band", self.lo, self.hi, self.sink, self.q_offset)
+
+    def c_struct(self) -> _lib.FlexMask:
+        m = _lib.FlexMask()
+        m.kind, m.lo, m.hi, m.sink, m.q_offset = self.kind, self.lo, self.hi, self.sink, self.q_offset
+        if self.bits is not None:
+            Bm, Hm, Qp, W = self.bits.shape
+            m.bits = self.bits.data_ptr()
+            m.bits_stride_b = 0 if Bm == 1 else Hm * Qp * W
+            m.bits_stride_h = 0 if Hm == 1 else Qp * W
+            m.bits_stride_q = W
+        return m
+
+    def __call__(self, b, h, q_idx, kv_idx):
+        if self.bits is not None:
+            return self.fn(b, h, q_idx, kv_idx)
+        d = q_idx + self.q_offset - kv_idx
+        r = (d >= self.lo)
+        if self.hi != INT_MAX:
+            r = r & ((d <= self.hi) | ((kv_idx + 0 * q_idx) <= self.sink))
+        return r
+
+    def __repr__(self):
+        if self.bits is not None:
+            return f"MaskMod({self.__name__}, bitmap {tuple(self.bits.shape)})"
+        return f"MaskMod({self.__name__}, lo={self.lo}, hi={self.hi}, sink={self.sink}, q_offset={self.q_offset})"
+
+
+def band_and(a: MaskMod, b: MaskMod) -> Optional[MaskMod]:
+    """Intersection of two band masks when it is again a band mask."""
+    if a.bits is not None or b.bits is not None or a.q_offset != b.q_offset:
+        return None
+    lo = max(a.lo, b.lo)
+    if a.hi == INT_MAX:
+        hi, sink = b.hi, b.sink
+    elif b.hi == INT_MAX:
+        hi, sink = a.hi, a.sink
+    elif a.sink == b.sink:
+        hi, sink = min(a.hi, b.hi), a.sink
+    elif a.hi == b.hi:
+        hi, sink = a.hi, min(a.sink, b.sink)
+    else:
+        return None
+    return MaskMod(lo, hi, sink, a.q_offset, name="and_mask")
+
+
+def band_or(a: MaskMod, b: MaskMod) -> Optional[MaskMod]:
+    """Union of two band masks when it is again a band mask."""
+    if a.bits is not None or b.bits is not None or a.q_offset != b.q_offset:
+        return None
+    if a.lo == INT_MIN and b.lo == INT_MIN:
+        return MaskMod(INT_MIN, max(a.hi, b.hi), max(a.sink, b.sink), a.q_offset, name="or_mask")
+    if a.lo == INT_MAX:
+        return b
+    if b.lo == INT_MAX:
+        return a
+    if (a.hi, a.sink) == (b.hi, b.sink):
+        return MaskMod(min(a.lo, b.lo), a.hi, a.sink, a.q_offset, name="or_mask")
+    return None
+
+
+def _pad128(n: int) -> int:
+    return (n + 127) // 128 * 128
+
+
+def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device) -> torch.Tensor:
+    """Evaluate a Python mask_mod (or a five-argument score_mod, which masks
+    where it returns -inf: flaxattention/core/blockmask.py:307-315) over the
+    whole index grid with device tensors.  bool [B,H,Q,KV]."""
+    b = torch.arange(B, dtype=torch.int32, device=device).reshape(B, 1, 1, 1)
+    h = torch.arange(H, dtype=torch.int32, device=device).reshape(1, H, 1, 1)
+    q = torch.arange(Q, dtype=torch.int32, device=device).reshape(1, 1, Q, 1)
+    kv = torch.arange(KV, dtype=torch.int32, device=device).reshape(1, 1, 1, KV)
+    if _get_mod_type(fn) == _ModificationType.SCORE_MOD:
+        out = fn(torch.zeros(B, H, Q, KV, device=device), b, h, q, kv)
+        m = ~torch.isneginf(torch.as_tensor(out, device=device))
+    else:
+        m = fn(b, h, q, kv)
+        if not torch.is_tensor(m):
+            m = torch.tensor(bool(m), device=device)
+    return m.to(device=device, dtype=torch.bool)
+
+
+def _fit_band(m2: torch.Tensor) -> Optional[MaskMod]:
+    """Given a [Q,KV] boolean matrix, find band parameters that reproduce it
+    exactly over the whole matrix, if any."""
+    Q, KV = m2.shape
+    dev = m2.device
+    q = torch.arange(Q, device=dev, dtype=torch.int64).reshape(Q, 1)
+    kv = torch.arange(KV, device=dev, dtype=torch.int64).reshape(1, KV)
+    d = q - kv
+    if not bool(m2.any()):
+        return MaskMod(INT_MAX, INT_MAX, -1, name="all_false")
+    lo = int(d[m2].min())
+    if lo <= -(KV - 1):
+        lo = INT_MIN
+    inside = d >= lo
+    hidden = inside & ~m2
+    cands = []
+    if not bool(hidden.any()):
+        cands.append((lo, INT_MAX, -1))
+    else:
+        hi = int(d[hidden].min()) - 1
+        sink = int(torch.broadcast_to(kv, d.shape)[hidden].min()) - 1
+        cands.append((lo, hi, sink))
+        cands.append((lo, hi, -1))
+    for lo_, hi_, sink_ in cands:
+        test = (d >= lo_) & ((d <= hi_) | (kv <= sink_))
+        if bool((test == m2).all()):
+            return MaskMod(lo_, hi_, sink_, name="band")
+    return None
+
+
+def pack_bits(mask: torch.Tensor) -> torch.Tensor:
+    """bool [..., KV] -> int32 words [..., ceil(KV/32)], bit (kv & 31) of word kv >> 5."""
+    *lead, KV = mask.shape
+    W = (KV + 31) // 32
+    if W * 32 != KV:
+        mask = torch.nn.functional.pad(mask, (0, W * 32 - KV))
+    m = mask.reshape(*lead, W, 32).to(torch.int64)
+    weights = (1 << torch.arange(32, device=mask.device, dtype=torch.int64))
+    words = (m * weights).sum(-1)
+    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words)
+    return words.to(torch.int32).contiguous()
+
+
+def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, device) -> MaskMod:
+    """Lower a mask_mod callable to a kernel functor that is exact on the
+    index range [0, pad128(Q)) x [0, pad128(KV)).  Tagged functors pass
+    through; any other callable is evaluated densely on the device once and
+    either recognised as a band mask (checked against every entry) or kept as
+    a packed bitmap."""
+    if fn is None:
+        return MaskMod(name="noop_mask")
+    if isinstance(fn, MaskMod) and fn.bits is None:
+        return fn
+    if isinstance(fn, MaskMod):
+        Bm, Hm, Qp, W = fn.bits.shape
+        if Qp >= _pad128(Q) and W * 32 >= _pad128(KV) and Bm in (1, B) and Hm in (1, H):
+            return fn
+        fn = fn.fn
+    Qp, KVp = _pad128(Q), _pad128(KV)
+    m = dense_mask_on_device(fn, B, H, Qp, KVp, device)
+    name = getattr(fn, "__name__", "mask_mod")
+    full_shape = torch.broadcast_shapes(m.shape, (1, 1, Qp, KVp))
+    m = torch.broadcast_to(m, full_shape)
+    bh_indep = bool((m == m[:1, :1]).all()) if (full_shape[0] > 1 or full_shape[1] > 1) else True
+    if bh_indep:
+        band = _fit_band(m[0, 0])
+        if band is not None:
+            band.__name__ = name
+            return band
+        m = m[:1, :1]
+    bits = pack_bits(m.contiguous())
+    return MaskMod(name=name, bits=bits, fn=fn)

@@ -1,0 +1,142 @@
+// Block-mask builder for gfx950.
+//
+// Replaces the dense [B,H,Q,KV] boolean mask + reshape/sum + argsort pipeline of
+// flaxattention/core/blockmask.py:277-322, 335-369, 57-64: the mask functor is
+// evaluated per tile in registers, each tile is classified empty / partial /
+// full, and the per-row ordered index lists are produced by a wave-level
+// stable partition (selected ids ascending, then the rest ascending -- the
+// order a stable descending argsort of a 0/1 row gives).  The dense mask is
+// never materialised.  All outputs are integers and bit-exact.
+#include "flex_common.cuh"
+
+namespace flex {
+
+constexpr int kClassifyThreads = 256;
+
+// One workgroup per tile.  flags: [B*H, nq, nkv] int8 for partial and full.
+__global__ __launch_bounds__(kClassifyThreads) void classify_tiles_kernel(
+    FlexMask mask, int H, int nq, int nkv, int qb, int kvb, int8_t* __restrict__ partial,
+    int8_t* __restrict__ full) {
+  const int ki = blockIdx.x, qi = blockIdx.y, bh = blockIdx.z;
+  const int b = bh / H, h = bh % H;
+  MaskEval visible(mask, b, h);
+  const int q0 = qi * qb, kv0 = ki * kvb;
+  const long long total = (long long)qb * kvb;
+  unsigned long long cnt = 0;
+  if (mask.kind == FLEX_MASK_BITS && (kvb % 32) == 0) {
+    // word-at-a-time: every aligned 32-bit word of a row lies inside the tile
+    const int words = kvb / 32;
+    const long long nwords = (long long)qb * words;
+    for (long long t = threadIdx.x; t < nwords; t += kClassifyThreads) {
+      int r = (int)(t / words), w = (int)(t % words);
+      uint32_t bits = visible.bits_bh[(int64_t)(q0 + r) * visible.stride_q + (kv0 >> 5) + w];
+      cnt += __popc(bits);
+    }
+  } else {
+    for (long long t = threadIdx.x; t < total; t += kClassifyThreads) {
+      int r = (int)(t / kvb), c = (int)(t % kvb);
+      cnt += visible(q0 + r, kv0 + c) ? 1u : 0u;
+    }
+  }
+  // workgroup reduction
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_xor(cnt, off, 64);
+  __shared__ unsigned long long wsum[kClassifyThreads / 64];
+  if ((threadIdx.x & 63) == 0) wsum[threadIdx.x >> 6] = cnt;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long s = 0;
+    for (int w = 0; w < kClassifyThreads / 64; w++) s += wsum[w];
+    size_t at = ((size_t)bh * nq + qi) * nkv + ki;
+    full[at] = (s == (unsigned long long)total) ? 1 : 0;
+    partial[at] = (s > 0 && s < (unsigned long long)total) ? 1 : 0;
+  }
+}
+
+// One wave per output row.  Reads flags[bh][r*row_stride + c*col_stride] for
+// c in [0, ncols) and writes num[bh][r] and idx[bh][r][0..ncols).
+__global__ __launch_bounds__(256) void order_rows_kernel(const int8_t* __restrict__ flags, int nrows,
+                                                         int ncols, long long mat_stride,
+                                                         int row_stride, int col_stride,
+                                                         int32_t* __restrict__ num,
+                                                         int32_t* __restrict__ idx, long long total_rows) {
+  const int lane = threadIdx.x & 63;
+  const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (row >= total_rows) return;
+  const long long bh = row / nrows;
+  const int r = (int)(row % nrows);
+  const int8_t* f = flags + bh * mat_stride + (long long)r * row_stride;
+  int count = 0;
+  for (int c0 = 0; c0 < ncols; c0 += 64) {
+    int c = c0 + lane;
+    bool sel = (c < ncols) && f[(long long)c * col_stride] != 0;
+    count += __popcll(__ballot(sel));
+  }
+  if (num && lane == 0) num[row] = count;
+  if (!idx) return;
+  int32_t* out = idx + row * ncols;
+  int before_sel = 0, before_uns = 0;
+  const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+  for (int c0 = 0; c0 < ncols; c0 += 64) {
+    int c = c0 + lane;
+    bool in = c < ncols;
+    bool sel = in && f[(long long)c * col_stride] != 0;
+    unsigned long long ms = __ballot(sel), mu = __ballot(in && !sel);
+    if (sel) out[before_sel + __popcll(ms & lt)] = c;
+    else if (in) out[count + before_uns + __popcll(mu & lt)] = c;
+    before_sel += __popcll(ms);
+    before_uns += __popcll(mu);
+  }
+}
+
+}  // namespace flex
+
+using namespace flex;
+
+extern "C" size_t flexattn_block_mask_workspace_bytes(int32_t B, int32_t H, int32_t nq, int32_t nkv) {
+  size_t n = (size_t)B * H * nq * nkv;
+  return 2 * ((n + 255) / 256 * 256);
+}
+
+void flex_set_error(const char* fmt, ...);
+
+extern "C" int flexattn_block_mask_build(const FlexMask* mask, int32_t B, int32_t H, int32_t nq,
+                                         int32_t nkv, int32_t qb, int32_t kvb, int32_t* kv_num,
+                                         int32_t* kv_idx, int32_t* full_kv_num, int32_t* full_kv_idx,
+                                         int32_t* q_num, int32_t* q_idx, int32_t* full_q_num,
+                                         int32_t* full_q_idx, void* workspace,
+                                         flexattn_stream_t stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!mask || !workspace) { flex_set_error("block_mask_build: null mask or workspace"); return 1; }
+  if (B <= 0 || H <= 0 || nq <= 0 || nkv <= 0 || qb <= 0 || kvb <= 0) {
+    flex_set_error("block_mask_build: non-positive size B=%d H=%d nq=%d nkv=%d qb=%d kvb=%d", B, H, nq, nkv, qb, kvb);
+    return 1;
+  }
+  if ((long long)B * H > 65535 || nq > 65535) {
+    flex_set_error("block_mask_build: grid too large (B*H=%lld, nq=%d; limit 65535)", (long long)B * H, nq);
+    return 1;
+  }
+  if (mask->kind == FLEX_MASK_BITS && !mask->bits) { flex_set_error("block_mask_build: bitmap mask without bits"); return 1; }
+  if (mask->kind != FLEX_MASK_BITS && mask->kind != FLEX_MASK_BAND) { flex_set_error("block_mask_build: unknown mask kind %d", mask->kind); return 1; }
+  size_t n = (size_t)B * H * nq * nkv;
+  int8_t* partial = (int8_t*)workspace;
+  int8_t* full = partial + (n + 255) / 256 * 256;
+  dim3 grid(nkv, nq, B * H);
+  hipLaunchKernelGGL(classify_tiles_kernel, grid, dim3(kClassifyThreads), 0, stream, *mask, H, nq, nkv, qb, kvb, partial, full);
+  const long long mat = (long long)nq * nkv;
+  auto order = [&](const int8_t* flags, bool transposed, int32_t* num, int32_t* idx) {
+    if (!num && !idx) return;
+    int nrows = transposed ? nkv : nq, ncols = transposed ? nq : nkv;
+    int rs = transposed ? 1 : nkv, cs = transposed ? nkv : 1;
+    long long total_rows = (long long)B * H * nrows;
+    int waves = 4;
+    long long blocks = (total_rows + waves - 1) / waves;
+    hipLaunchKernelGGL(order_rows_kernel, dim3((unsigned)blocks), dim3(64 * waves), 0, stream, flags, nrows, ncols, mat, rs, cs, num, idx, total_rows);
+  };
+  order(partial, false, kv_num, kv_idx);
+  order(full, false, full_kv_num, full_kv_idx);
+  order(partial, true, q_num, q_idx);
+  order(full, true, full_q_num, full_q_idx);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { flex_set_error("block_mask_build: launch failed: %s", hipGetErrorString(e)); return 2; }
+  return 0;
+}

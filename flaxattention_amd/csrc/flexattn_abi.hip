@@ -1,0 +1,129 @@
+// extern "C" entry points: validation, dispatch, error reporting.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include "flex_common.cuh"
+
+static thread_local char g_err[512] = "";
+
+void flex_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+// implemented in the kernel translation units
+int flex_generic_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+int flex_generic_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
+                     void* dq, void* dk, void* dv, float* delta, hipStream_t s);
+bool flex_mfma_fwd_supported(const FlexAttnParams& p);
+int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+bool flex_mfma_bwd_supported(const FlexAttnParams& p);
+size_t flex_mfma_bwd_workspace(const FlexAttnParams& p);
+int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                  const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
+bool flex_decode_supported(const FlexAttnParams& p);
+int flex_decode_default_splits(const FlexAttnParams& p);
+size_t flex_decode_workspace(const FlexAttnParams& p, int splits);
+int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
+                       void* workspace, hipStream_t s);
+void flex_mfma_tiles(int dtype, int D, int Dv, int* qb, int* kvb);
+
+static int validate(const FlexAttnParams* p, const char* who) {
+  if (!p) { flex_set_error("%s: null params", who); return 1; }
+  if (p->dtype < FLEX_F32 || p->dtype > FLEX_BF16) { flex_set_error("%s: unknown dtype %d", who, p->dtype); return 1; }
+  if (p->B <= 0 || p->Hq <= 0 || p->Hkv <= 0 || p->Lq <= 0 || p->Lkv <= 0 || p->D <= 0 || p->Dv <= 0) {
+    flex_set_error("%s: non-positive size B=%d Hq=%d Hkv=%d Lq=%d Lkv=%d D=%d Dv=%d", who, p->B, p->Hq, p->Hkv, p->Lq, p->Lkv, p->D, p->Dv);
+    return 1;
+  }
+  if (p->Hq % p->Hkv != 0) { flex_set_error("%s: Hq=%d is not a multiple of Hkv=%d", who, p->Hq, p->Hkv); return 1; }
+  if (p->Dv > p->D) { flex_set_error("%s: Dv=%d must be <= D=%d", who, p->Dv, p->D); return 1; }
+  if (p->score.kind < FLEX_SCORE_IDENTITY || p->score.kind > FLEX_SCORE_REL_BIAS) { flex_set_error("%s: unknown score_mod kind %d", who, p->score.kind); return 1; }
+  if (p->score.kind == FLEX_SCORE_ALIBI && p->score.i0 <= 0) { flex_set_error("%s: ALiBi needs the head count in i0", who); return 1; }
+  if (p->score.kind == FLEX_SCORE_TANH_SOFTCAP && !(p->score.p0 > 0.f)) { flex_set_error("%s: tanh soft-cap needs cap > 0", who); return 1; }
+  if (p->mask.kind != FLEX_MASK_BAND && p->mask.kind != FLEX_MASK_BITS) { flex_set_error("%s: unknown mask kind %d", who, p->mask.kind); return 1; }
+  if (p->mask.kind == FLEX_MASK_BITS && !p->mask.bits) { flex_set_error("%s: bitmap mask without bits", who); return 1; }
+  const FlexTileLists& t = p->tiles;
+  if (t.kv_num) {
+    if (!t.kv_idx || !t.full_kv_num || !t.full_kv_idx) { flex_set_error("%s: tile lists need kv_idx, full_kv_num and full_kv_idx", who); return 1; }
+    if (t.q_block <= 0 || t.kv_block <= 0 || (int64_t)t.n_q_blocks * t.q_block < p->Lq || (int64_t)t.n_kv_blocks * t.kv_block < p->Lkv) {
+      flex_set_error("%s: tile lists (%d x %d blocks of %d x %d) do not cover Lq=%d, Lkv=%d", who, t.n_q_blocks, t.n_kv_blocks, t.q_block, t.kv_block, p->Lq, p->Lkv);
+      return 1;
+    }
+  }
+  return 0;
+}
+
+static int check_launch(const char* who) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { flex_set_error("%s: kernel launch failed: %s", who, hipGetErrorString(e)); return 2; }
+  return 0;
+}
+
+extern "C" int flexattn_abi_version(void) { return 1; }
+extern "C" const char* flexattn_last_error(void) { return g_err; }
+
+extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t* qb, int32_t* kvb) {
+  int a = 0, b = 0;
+  flex_mfma_tiles(dtype, D, Dv, &a, &b);
+  if (qb) *qb = a;
+  if (kvb) *kvb = b;
+  return 0;
+}
+
+extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) { return 0; }
+
+extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
+                            void* workspace, flexattn_stream_t stream) {
+  if (int rc = validate(p, "flexattn_fwd")) return rc;
+  if (!q || !k || !v || !o) { flex_set_error("flexattn_fwd: null tensor pointer"); return 1; }
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (!(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)) && flex_mfma_fwd_supported(*p)) rc = flex_mfma_fwd(*p, q, k, v, o, lse2, s);
+  else rc = flex_generic_fwd(*p, q, k, v, o, lse2, s);
+  if (rc) return rc;
+  return check_launch("flexattn_fwd");
+}
+
+static size_t delta_bytes(const FlexAttnParams* p) { return ((size_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256; }
+
+extern "C" size_t flexattn_bwd_workspace_bytes(const FlexAttnParams* p) {
+  if (!p) return 0;
+  size_t n = delta_bytes(p);
+  if (!(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)) && flex_mfma_bwd_supported(*p)) n += flex_mfma_bwd_workspace(*p);
+  return n;
+}
+
+extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, const void* o,
+                            const float* lse2, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
+                            flexattn_stream_t stream) {
+  if (int rc = validate(p, "flexattn_bwd")) return rc;
+  if (!q || !k || !v || !o || !lse2 || !d_o || !dq || !dk || !dv || !workspace) { flex_set_error("flexattn_bwd: null pointer"); return 1; }
+  hipStream_t s = (hipStream_t)stream;
+  int rc;
+  if (!(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)) && flex_mfma_bwd_supported(*p)) rc = flex_mfma_bwd(*p, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s);
+  else rc = flex_generic_bwd(*p, q, k, v, lse2, d_o, dq, dk, dv, (float*)workspace, s);
+  if (rc) return rc;
+  return check_launch("flexattn_bwd");
+}
+
+extern "C" size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32_t num_splits) {
+  if (!p) return 0;
+  if (num_splits <= 0) num_splits = flex_decode_default_splits(*p);
+  return flex_decode_workspace(*p, num_splits);
+}
+
+extern "C" int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
+                               int32_t num_splits, void* workspace, flexattn_stream_t stream) {
+  if (int rc = validate(p, "flexattn_decode")) return rc;
+  if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
+  if (!flex_decode_supported(*p)) {
+    flex_set_error("flexattn_decode: needs fp16/bf16, D == Dv in {64,128}, Lq <= 64 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
+    return 1;
+  }
+  if (num_splits <= 0) num_splits = flex_decode_default_splits(*p);
+  int rc = flex_decode_launch(*p, q, k, v, o, lse2, num_splits, workspace, (hipStream_t)stream);
+  if (rc) return rc;
+  return check_launch("flexattn_decode");
+}

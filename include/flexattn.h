@@ -1,0 +1,167 @@
+/*
+ * flexattn.h -- C ABI of the MI355X (gfx950) FlexAttention engine.
+ *
+ * The reference (zinccat/flaxattention) has no native boundary: its surface is
+ * Python (flax_attention, flax_attention_pallas, create_block_mask) over
+ * jax.custom_vjp.  Each entry point below names the reference function whose
+ * device work it replaces.  All tensor pointers are DEVICE pointers; every
+ * call only enqueues work on `stream` and returns without synchronising.
+ * Return value: 0 on success, non-zero on error with a thread-local message
+ * available from flexattn_last_error().  No entry point allocates memory:
+ * scratch is passed in by the caller and sized by the *_workspace_bytes
+ * helpers.  Entry points are re-entrant.
+ */
+#ifndef FLEXATTN_H_
+#define FLEXATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* flexattn_stream_t; /* a hipStream_t */
+
+enum FlexDType { FLEX_F32 = 0, FLEX_F16 = 1, FLEX_BF16 = 2 };
+
+/* score_mod functors: the scalar functions of (score, b, h, q_idx, kv_idx)
+ * that flaxattention/core/common.py:7 types as _score_mod_signature. */
+enum FlexScoreKind {
+  FLEX_SCORE_IDENTITY = 0,     /* flaxattention/core/attention.py:109-116 */
+  FLEX_SCORE_CHECKERBOARD = 1, /* examples/benchmark.py:16-22; i0 = 0: parity of
+                                  (kv_idx - q_idx), i0 = 1: parity of kv_idx;
+                                  p0 multiplies even entries, p1 odd entries */
+  FLEX_SCORE_ALIBI = 2,        /* flaxattention/mods/alibi.py:15-18:
+                                  score + p0*(q_idx-kv_idx)*exp2(-(h+1)*8/i0) */
+  FLEX_SCORE_TANH_SOFTCAP = 3, /* p0 * tanh(score / p0) */
+  FLEX_SCORE_REL_BIAS = 4      /* score + p0 * (kv_idx - q_idx) */
+};
+
+typedef struct FlexScoreMod {
+  int32_t kind;
+  float p0, p1;
+  int32_t i0, i1;
+} FlexScoreMod;
+
+/* mask_mod functors (flaxattention/core/common.py:8).  FLEX_MASK_BAND is a
+ * canonical form that covers noop_mask (blockmask.py:20-27), causal_mask
+ * (masks/causal.py:4-5), generate_sliding_window (masks/sliding_window.py:
+ * 7-22), generate_attention_sink (masks/attention_sink.py:6-24) and their
+ * and_masks combinations:
+ *     d = q_idx + q_offset - kv_idx
+ *     visible = (d >= lo) && (d <= hi || kv_idx <= sink)
+ * FLEX_MASK_BITS reads a packed bitmap produced from an arbitrary Python
+ * callable: bit (kv & 31) of word bits[b*sb + h*sh + q*sq + (kv >> 5)].  */
+enum FlexMaskKind { FLEX_MASK_BAND = 0, FLEX_MASK_BITS = 1 };
+
+typedef struct FlexMask {
+  int32_t kind;
+  int32_t lo, hi, sink, q_offset;
+  int32_t pad_;
+  const uint32_t* bits;
+  int64_t bits_stride_b, bits_stride_h, bits_stride_q; /* in 32-bit words */
+} FlexMask;
+
+/* numerics switches (OR-ed into FlexAttnParams.flags) */
+enum FlexFlags {
+  FLEX_ROUND_S = 1,      /* round Q.K^T through the input dtype before scaling
+                            (attention.py:27 computes the product in that dtype) */
+  FLEX_STRICT = 2,       /* generic kernels only: also round the normalised P,
+                            dP and dS through the input dtype (attention.py:105
+                            and its transposes) */
+  FLEX_FORCE_GENERIC = 4 /* never use the MFMA kernels */
+};
+
+/* Ordered tile lists in the layout of BlockMask.kv_num_blocks / kv_indices /
+ * full_kv_* (blockmask.py:72-119), at the granularity (q_block, kv_block).
+ * A NULL kv_num means "visit every tile and evaluate the mask in each".
+ * Counts are [Bm, Hm, n_q_blocks], indices [Bm, Hm, n_q_blocks, n_kv_blocks];
+ * Bm/Hm may be 1 (broadcast) -- give stride 0.  The transposed lists
+ * (q_num / q_idx, per kv block) drive the dK/dV kernel.  */
+typedef struct FlexTileLists {
+  const int32_t* kv_num;
+  const int32_t* kv_idx;
+  const int32_t* full_kv_num;
+  const int32_t* full_kv_idx;
+  const int32_t* q_num;
+  const int32_t* q_idx;
+  const int32_t* full_q_num;
+  const int32_t* full_q_idx;
+  int32_t q_block, kv_block;
+  int32_t n_q_blocks, n_kv_blocks;
+  int64_t stride_b, stride_h; /* in rows of the count arrays */
+} FlexTileLists;
+
+typedef struct FlexAttnParams {
+  int32_t dtype; /* FlexDType of q, k, v, o, do, dq, dk, dv */
+  int32_t B, Hq, Hkv, Lq, Lkv, D, Dv;
+  /* element strides of the (batch, head, position) axes; the feature axis is
+   * contiguous.  [B,H,L,D] and [B,L,H,D] (flax_attention_pallas bhln=False,
+   * attention.py:243-246) are both expressible. */
+  int64_t q_stride[3], k_stride[3], v_stride[3], o_stride[3];
+  float scale;
+  int32_t flags;
+  FlexScoreMod score;
+  FlexMask mask;
+  FlexTileLists tiles;
+} FlexAttnParams;
+
+int flexattn_abi_version(void);
+const char* flexattn_last_error(void);
+
+/* Tile sizes the fused kernels want their FlexTileLists built at for this
+ * problem (0/0 when only the generic kernels apply and lists are ignored). */
+int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv,
+                             int32_t* q_block, int32_t* kv_block);
+
+/* Block-mask builder.  Replaces create_block_mask -> _create_block_mask_inner
+ * -> create_mask / _convert_mask_to_block_mask -> _dense_to_ordered
+ * (flaxattention/core/blockmask.py:419-455, 400-416, 277-322, 335-369, 57-64)
+ * and the transposes of BlockMask.from_kv_blocks (121-164).  q_len / kv_len
+ * are the padded lengths n_q_blocks*q_block / n_kv_blocks*kv_block; the mask is
+ * evaluated on that whole index range (blockmask.py:440-444).  Outputs are
+ * int32: counts [B,H,nq], indices [B,H,nq,nkv]; q_* are [B,H,nkv] and
+ * [B,H,nkv,nq].  Any output pointer may be NULL.  `workspace` holds
+ * flexattn_block_mask_workspace_bytes() bytes.  */
+size_t flexattn_block_mask_workspace_bytes(int32_t B, int32_t H, int32_t n_q_blocks, int32_t n_kv_blocks);
+int flexattn_block_mask_build(const FlexMask* mask, int32_t B, int32_t H,
+                              int32_t n_q_blocks, int32_t n_kv_blocks,
+                              int32_t q_block, int32_t kv_block,
+                              int32_t* kv_num, int32_t* kv_idx,
+                              int32_t* full_kv_num, int32_t* full_kv_idx,
+                              int32_t* q_num, int32_t* q_idx,
+                              int32_t* full_q_num, int32_t* full_q_idx,
+                              void* workspace, flexattn_stream_t stream);
+
+/* Forward.  Replaces math_attention (flaxattention/core/attention.py:67-106)
+ * behind flax_attention (169-218) and mha_forward_kernel / _mha_forward
+ * (flaxattention/kernel/attention.py:34-149, 260-335) behind
+ * flax_attention_pallas (attention.py:220-312).  o: same layout family as q
+ * with Dv features; lse2: [B,Hq,Lq] fp32 base-2 log-sum-exp (-inf on rows with
+ * no visible key), may be NULL.  */
+size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p);
+int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v,
+                 void* o, float* lse2, void* workspace, flexattn_stream_t stream);
+
+/* Backward.  Replaces jax.grad through math_attention (the reference's pure
+ * path) and _preprocess_backward / mha_backward_kernel / _mha_backward
+ * (flaxattention/kernel/attention.py:338-650).  P is recomputed from lse2.
+ * dq/dk/dv are contiguous [B,H,L,D] tensors of the input dtype.  */
+size_t flexattn_bwd_workspace_bytes(const FlexAttnParams* p);
+int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* k, const void* v,
+                 const void* o, const float* lse2, const void* d_o,
+                 void* dq, void* dk, void* dv, void* workspace, flexattn_stream_t stream);
+
+/* Split-KV decode for short queries (Lq <= 64).  Replaces the same reference
+ * functions as flexattn_fwd for the decode shapes of
+ * examples/benchmark_decoding.py:29-33.  num_splits <= 0 picks a default.  */
+size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32_t num_splits);
+int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const void* v,
+                    void* o, float* lse2, int32_t num_splits, void* workspace,
+                    flexattn_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLEXATTN_H_ */

