@@ -36,7 +36,9 @@ def close(got, want, dtype, what, fused=False, scale_maxabs=False):
     ma, rl = tol_for(dtype, fused)
     got = got.detach().cpu()
     a, r = max_abs(got, want), rel_l2(got, want)
-    if scale_maxabs:  # large-magnitude gradients: max-abs relative to the largest entry
+    if scale_maxabs or (fused and dtype == torch.bfloat16):
+        # one bf16 ulp is 3.1e-2 for |x| in [4, 8): the absolute bound is scaled by
+        # the largest reference entry wherever values of that size occur
         ma = ma * max(1.0, want.abs().max().item())
     print(f"  {what}: max-abs {a:.3e} rel-L2 {r:.3e} (tol {ma:.1e} / {rl:.1e})", flush=True)
     assert a <= ma, f"{what}: max-abs {a} > {ma}"
@@ -216,3 +218,61 @@ def test_errors(dev):
         fa.flax_attention(q.cpu(), k.cpu(), v.cpu(), enable_gqa=True)   # no CPU fallback
     with pytest.raises(RuntimeError):
         fa.and_masks(causal_mask, 3)
+
+
+# ---- fused MFMA kernels (default path for fp16 / bf16, D in {64, 128}) ----
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name,score,oscore", SCORES, ids=[s[0] for s in SCORES])
+def test_fused_scores(dev, dtype, D, name, score, oscore):
+    print(f"case fused {name} {dtype} D{D}", flush=True)
+    big = name == "alibi_ref"
+    run(dev, dtype, 2, 4, 4, 256, 320, D, score=score, oscore=oscore, mask=causal_mask, omask=o_causal_mask,
+        strict=False, scale_maxabs=big)
+
+
+@pytest.mark.parametrize("name,mask,omask", MASKS, ids=[m[0] for m in MASKS])
+def test_fused_masks(dev, name, mask, omask):
+    print(f"case fused mask {name}", flush=True)
+    run(dev, torch.float16, 1, 2, 2, 384, 448, 64, mask=mask, omask=omask, strict=False)
+
+
+def test_fused_no_mask_checkerboard_config2_small(dev):
+    # benchmark configuration 2 at reduced batch: fp16, checkerboard, no mask
+    run(dev, torch.float16, 1, 2, 2, 2048, 2048, 64, score=checkerboard, oscore=o_checkerboard, strict=False)
+
+
+def test_fused_ragged_gqa(dev):
+    run(dev, torch.float16, 2, 8, 2, 77, 203, 64, mask=causal_mask, omask=o_causal_mask,
+        score=generate_alibi_bias(8, -1.0), oscore=o_alibi_config(8), strict=False)
+    run(dev, torch.bfloat16, 1, 4, 1, 300, 131, 128, strict=False)
+
+
+def test_fused_bitmap_mask_dead_rows(dev):
+    def weird(b, h, q_idx, kv_idx):
+        return ((q_idx * 7 + kv_idx * 3 + h) % 11 < 6) & (q_idx % 5 != 0)
+    run(dev, torch.float16, 2, 3, 3, 200, 260, 64, mask=weird, omask=weird, strict=False)
+
+    def doc_mask(b, h, q_idx, kv_idx):
+        return (q_idx // 192) == (kv_idx // 192)
+    run(dev, torch.float16, 1, 2, 2, 768, 768, 64, mask=doc_mask, omask=doc_mask, strict=False)
+
+
+def test_fused_fully_masked(dev):
+    def fullmask(b, h, q_idx, kv_idx):
+        return False
+    out = run(dev, torch.float16, 1, 2, 2, 128, 128, 64, mask=fullmask, omask=o_full_masked, strict=False)
+    assert torch.count_nonzero(out).item() == 0
+
+
+def test_fused_round_s_off_matches_excess_precision_oracle(dev):
+    q, k, v = seeded_qkv(1, 2, 2, 512, 512, 64, torch.float16)
+    want = ref_attention(q, k, v, o_checkerboard, None, strict=False)
+    out = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=checkerboard, kernel_options={"round_s": False})
+    close(out, want, torch.float16, "O (no S rounding vs non-strict oracle)", fused=True)
+
+
+def test_fused_decode_shapes_through_prefill_kernel(dev):
+    for ql in (1, 16, 64):
+        run(dev, torch.float16, 2, 4, 4, ql, 1024, 64, score=generate_alibi_bias(4, -1.0), oscore=o_alibi_config(4),
+            mask=offset_causal_mask(1024 - ql), omask=o_offset_causal(1024 - ql), strict=False, grad=False)
