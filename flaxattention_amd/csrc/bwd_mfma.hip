@@ -1,6 +1,450 @@
-#include "flex_common.cuh"
+// Fused flash-attention backward for gfx950 (fp16 / bf16, D = Dv in {64, 128}).
+//
+// Takes the place of _preprocess_backward + mha_backward_kernel
+// (flaxattention/kernel/attention.py:338-553) and of jax.grad through the dense
+// path.  P is recomputed from the saved base-2 log-sum-exp.  Two kernels:
+//
+//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 64
+//                  (the forward's schedule).  Transposed products keep one query
+//                  row per lane, so lse and delta are per-lane scalars:
+//                    S^T = K.Q^T,  dP^T = V.dO^T,  dS^T = P^T o (dP^T - delta) * g,
+//                    dQ^T += K^T.dS^T.
+//                  Also produces delta_i = sum_d O_id dO_id for the second kernel.
+//  bwd_dkv_kernel  one workgroup per 64 key rows, sweeping query tiles of 128
+//                  from the transposed tile lists.  Here a lane owns one key
+//                  row: S = Q.K^T, dP = dO.V^T, dV^T += dO^T.P, dK^T += Q^T.dS.
+//                  Waves 0/1 and 2/3 split the query tile and are summed through
+//                  LDS at the end.  With GQA the workgroup loops over the query
+//                  heads of its group.
+#include "mfma_common.cuh"
+
+namespace flex {
+
+constexpr int kBM = 128;  // query tile (list granularity)
+constexpr int kBN = 64;   // key tile (list granularity)
+
+template <typename T, int D, int KIND, bool ROUND_S>
+__global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                      const T* __restrict__ k, const T* __restrict__ v,
+                                                      const T* __restrict__ o, const float* __restrict__ lse2,
+                                                      const T* __restrict__ d_o, T* __restrict__ dq,
+                                                      float* __restrict__ delta_out) {
+  typedef typename Frag<T>::vec8 vec8;
+  constexpr int BM = kBM, BN = kBN;
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
+  __shared__ __align__(16) T Ks[BN * ROWE];
+  __shared__ __align__(16) T Vs[BN * ROWE];
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
+  const int nqt = (p.Lq + BM - 1) / BM;
+  const int total = nqt * p.Hq * p.B;
+  const int wid = xcd_remap(blockIdx.x, total);
+  const int qt = nqt - 1 - (wid % nqt);
+  const int bh = wid / nqt;
+  const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int q_row = qt * BM + w * 32 + i32;
+  const int q_ld = min(q_row, p.Lq - 1);
+  const int64_t row_id = ((int64_t)b * p.Hq + h) * p.Lq + q_ld;
+
+  vec8 qf[DS], dof[DS];
+  float dpart = 0.f;
+  {
+    const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
+    const T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_ld * p.o_stride[2] + 8 * g;
+    const T* dop = d_o + row_id * D + 8 * g;  // dO is contiguous [B,Hq,Lq,D]
+#pragma unroll
+    for (int s = 0; s < DS; s++) {
+      qf[s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+      dof[s] = *reinterpret_cast<const vec8*>(dop + 16 * s);
+      vec8 of = *reinterpret_cast<const vec8*>(op + 16 * s);
+#pragma unroll
+      for (int e = 0; e < 8; e++) dpart = fmaf((float)of[e], (float)dof[s][e], dpart);
+    }
+  }
+  const float delta = xhalf_sum(dpart);
+  if (q_row < p.Lq && g == 0) delta_out[row_id] = delta;
+  float lse = lse2[row_id];
+  if (lse == -INFINITY) lse = INFINITY;  // row without visible keys: P = 0
+
+  const FlexTileLists& tl = p.tiles;
+  const int32_t* full_idx = nullptr;
+  const int32_t* part_idx = nullptr;
+  int n_full, n_part = 0;
+  if (tl.kv_num) {
+    const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
+    n_full = tl.full_kv_num[row];
+    n_part = tl.kv_num[row];
+    full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
+    part_idx = tl.kv_idx + row * tl.n_kv_blocks;
+  } else {
+    n_full = (p.Lkv + BN - 1) / BN;
+  }
+  const int nt = n_full + n_part;
+  auto tile_at = [&](int it) -> int {
+    if (!full_idx) return it;
+    return it < n_full ? full_idx[it] : part_idx[it - n_full];
+  };
+
+  const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
+  const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
+  const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
+  uint4 kreg[NLD], vreg[NLD];
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      int kv = kv0 + r;
+      if (kv < p.Lkv) {
+        kreg[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)kv * ks2 + cc * 8);
+        vreg[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)kv * vs2 + cc * 8);
+      } else {
+        kreg[j] = make_uint4(0, 0, 0, 0);
+        vreg[j] = make_uint4(0, 0, 0, 0);
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      *reinterpret_cast<uint4*>(Ks + r * ROWE + cc * 8) = kreg[j];
+      *reinterpret_cast<uint4*>(Vs + r * ROWE + cc * 8) = vreg[j];
+    }
+  };
+
+  Score2<KIND> sm;
+  sm.init(p.score, p.scale, h);
+  Mask2 visible(p.mask, b, h, p.Lkv);
+  float16_t dqacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dqacc[db][r] = 0.f;
+
+  if (nt > 0) load_tile(tile_at(0) * BN);
+  for (int it = 0; it < nt; it++) {
+    const int kv0 = tile_at(it) * BN;
+    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
+    store_tile();
+    __syncthreads();
+    if (it + 1 < nt) load_tile(tile_at(it + 1) * BN);
+
+    float16_t sacc[2], dpacc[2];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) { sacc[nb][r] = 0.f; dpacc[nb][r] = 0.f; }
+      const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+      const T* vp = Vs + (nb * 32 + i32) * ROWE + 8 * g;
+#pragma unroll
+      for (int s = 0; s < DS; s++) {
+        sacc[nb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + 16 * s), qf[s], sacc[nb]);
+        dpacc[nb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + 16 * s), dof[s], dpacc[nb]);
+      }
+    }
+    vec8 dsf[4];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      const int kvb = kv0 + nb * 32 + 4 * g;
+      sm.tile(q_row, kvb);
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        float s = sacc[nb][r];
+        if (ROUND_S) s = round_through<T>(s);
+        float x = sm.apply(s, acc_row(r));
+        if (masked) x = visible(q_row, kvb + acc_row(r)) ? x : -INFINITY;
+        float pr = fast_exp2(x - lse);
+        float ds = pr * (dpacc[nb][r] - delta) * (sm.grad(s, acc_row(r)) * p.scale);
+        dsf[2 * nb + r / 8][r % 8] = (T)ds;
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < 4; t++) {
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const T* kp = Ks + (16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+        short4_t lo = lds_read_tr(kp);
+        short4_t hi = lds_read_tr(kp + 8 * ROWE);
+        dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[t], dqacc[db]);
+      }
+    }
+    __syncthreads();
+  }
+
+  if (q_row < p.Lq) {
+    T* op = dq + row_id * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int rr = 0; rr < 4; rr++) {
+        union { T e[4]; uint2 u; } pk;
+#pragma unroll
+        for (int e = 0; e < 4; e++) pk.e[e] = (T)dqacc[db][4 * rr + e];
+        *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
+      }
+  }
+}
+
+extern __shared__ __align__(16) unsigned char bwd_smem[];
+
+template <typename T, int D, int KIND, bool ROUND_S>
+__global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                       const T* __restrict__ k, const T* __restrict__ v,
+                                                       const float* __restrict__ lse2,
+                                                       const float* __restrict__ delta,
+                                                       const T* __restrict__ d_o, T* __restrict__ dk,
+                                                       T* __restrict__ dv) {
+  typedef typename Frag<T>::vec8 vec8;
+  constexpr int BM = kBM, BN = kBN;
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / 256;
+  T* Qs = reinterpret_cast<T*>(bwd_smem);
+  T* Os = Qs + BM * ROWE;
+  float* lse_s = reinterpret_cast<float*>(Os + BM * ROWE);
+  float* del_s = lse_s + BM;
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
+  const int wk = w & 1, wq = w >> 1;
+  const int nkt = (p.Lkv + BN - 1) / BN;
+  const int total = nkt * p.Hkv * p.B;
+  const int wid = xcd_remap(blockIdx.x, total);
+  const int kt = wid % nkt;  // early key tiles see the most queries under causal masks
+  const int bh = wid / nkt;
+  const int hk = bh % p.Hkv, b = bh / p.Hkv, G = p.Hq / p.Hkv;
+  const int kv_col = kt * BN + wk * 32 + i32;
+  const int kv_ld = min(kv_col, p.Lkv - 1);
+
+  vec8 kf[DS], vf[DS];
+  {
+    const T* kp = k + b * p.k_stride[0] + hk * p.k_stride[1] + (int64_t)kv_ld * p.k_stride[2] + 8 * g;
+    const T* vp = v + b * p.v_stride[0] + hk * p.v_stride[1] + (int64_t)kv_ld * p.v_stride[2] + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DS; s++) {
+      kf[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+      vf[s] = *reinterpret_cast<const vec8*>(vp + 16 * s);
+    }
+  }
+  float16_t dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; db++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+
+  const FlexTileLists& tl = p.tiles;
+  Score2<KIND> sm;
+
+  for (int gi = 0; gi < G; gi++) {
+    const int h = hk * G + gi;
+    sm.init(p.score, p.scale, h);
+    Mask2 visible(p.mask, b, h, p.Lkv);
+    const int32_t* full_idx = nullptr;
+    const int32_t* part_idx = nullptr;
+    int n_full, n_part = 0;
+    if (tl.kv_num) {
+      const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_kv_blocks + kt;
+      n_full = tl.full_q_num[row];
+      n_part = tl.q_num[row];
+      full_idx = tl.full_q_idx + row * tl.n_q_blocks;
+      part_idx = tl.q_idx + row * tl.n_q_blocks;
+    } else {
+      n_full = (p.Lq + BM - 1) / BM;
+    }
+    const int nt = n_full + n_part;
+    const T* qbase = q + b * p.q_stride[0] + h * p.q_stride[1];
+    const int64_t rows0 = ((int64_t)b * p.Hq + h) * p.Lq;
+    const T* dobase = d_o + rows0 * D;
+
+    for (int it = 0; it < nt; it++) {
+      const int qtile = full_idx ? (it < n_full ? full_idx[it] : part_idx[it - n_full]) : it;
+      const int q0 = qtile * BM;
+      const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
+      __syncthreads();  // previous tile fully consumed
+#pragma unroll
+      for (int j = 0; j < NLD; j++) {
+        int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+        uint4 a = make_uint4(0, 0, 0, 0), d4 = make_uint4(0, 0, 0, 0);
+        if (q0 + r < p.Lq) {
+          a = *reinterpret_cast<const uint4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
+          d4 = *reinterpret_cast<const uint4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
+        }
+        *reinterpret_cast<uint4*>(Qs + r * ROWE + cc * 8) = a;
+        *reinterpret_cast<uint4*>(Os + r * ROWE + cc * 8) = d4;
+      }
+      if (tid < BM) {
+        float l = INFINITY, dl = 0.f;
+        if (q0 + tid < p.Lq) {
+          l = lse2[rows0 + q0 + tid];
+          dl = delta[rows0 + q0 + tid];
+          if (l == -INFINITY) l = INFINITY;
+        }
+        lse_s[tid] = l;
+        del_s[tid] = dl;
+      }
+      __syncthreads();
+
+      const int qbase_w = wq * 64;
+      float16_t sacc[2], dpacc[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) { sacc[mb][r] = 0.f; dpacc[mb][r] = 0.f; }
+        const T* qp = Qs + (qbase_w + mb * 32 + i32) * ROWE + 8 * g;
+        const T* op = Os + (qbase_w + mb * 32 + i32) * ROWE + 8 * g;
+#pragma unroll
+        for (int s = 0; s < DS; s++) {
+          sacc[mb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + 16 * s), kf[s], sacc[mb]);
+          dpacc[mb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + 16 * s), vf[s], dpacc[mb]);
+        }
+      }
+      vec8 pf[4], dsf[4];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+        const int ql = qbase_w + mb * 32 + 4 * g;  // local row of register 0
+        sm.tileT(q0 + ql, kv_col);
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+          const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
+          const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int r = 4 * rr + e;
+            float s = sacc[mb][r];
+            if (ROUND_S) s = round_through<T>(s);
+            float x = sm.apply(s, acc_row(r));
+            if (masked) {
+              const int qi = q0 + ql + acc_row(r);
+              x = (qi < p.Lq && visible(qi, kv_col)) ? x : -INFINITY;
+            }
+            float pr = fast_exp2(x - l4[e]);
+            float ds = pr * (dpacc[mb][r] - d4[e]) * (sm.grad(s, acc_row(r)) * p.scale);
+            pf[2 * mb + r / 8][r % 8] = (T)pr;
+            dsf[2 * mb + r / 8][r % 8] = (T)ds;
+          }
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < 4; t++) {
+#pragma unroll
+        for (int db = 0; db < DB; db++) {
+          const int off = (qbase_w + 16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+          vec8 a_do = join8<vec8>(lds_read_tr(Os + off), lds_read_tr(Os + off + 8 * ROWE));
+          dvacc[db] = Frag<T>::mfma(a_do, pf[t], dvacc[db]);
+          vec8 a_q = join8<vec8>(lds_read_tr(Qs + off), lds_read_tr(Qs + off + 8 * ROWE));
+          dkacc[db] = Frag<T>::mfma(a_q, dsf[t], dkacc[db]);
+        }
+      }
+    }
+  }
+
+  // sum the two query halves (waves wq = 0 and 1 of the same key block) through LDS
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(bwd_smem);  // [2 key blocks][2*DB*16 regs][64 lanes]
+  if (wq == 1) {
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        red[((wk * 2 * DB + db) * 16 + r) * 64 + lane] = dkacc[db][r];
+        red[((wk * 2 * DB + DB + db) * 16 + r) * 64 + lane] = dvacc[db][r];
+      }
+  }
+  __syncthreads();
+  if (wq == 0 && kv_col < p.Lkv) {
+    const int64_t row_id = ((int64_t)b * p.Hkv + hk) * p.Lkv + kv_col;
+    T* dkp = dk + row_id * D + 4 * g;
+    T* dvp = dv + row_id * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int rr = 0; rr < 4; rr++) {
+        union { T e[4]; uint2 u; } pk, pv;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = 4 * rr + e;
+          pk.e[e] = (T)(dkacc[db][r] + red[((wk * 2 * DB + db) * 16 + r) * 64 + lane]);
+          pv.e[e] = (T)(dvacc[db][r] + red[((wk * 2 * DB + DB + db) * 16 + r) * 64 + lane]);
+        }
+        *reinterpret_cast<uint2*>(dkp + 32 * db + 8 * rr) = pk.u;
+        *reinterpret_cast<uint2*>(dvp + 32 * db + 8 * rr) = pv.u;
+      }
+  }
+}
+
+template <int D, typename T> constexpr size_t dkv_smem() {
+  size_t tiles = (size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float);
+  size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
+  return tiles > red ? tiles : red;
+}
+
+template <typename T, int D, int KIND, bool RS>
+static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                      const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
+  const int nqt = (p.Lq + kBM - 1) / kBM, nkt = (p.Lkv + kBN - 1) / kBN;
+  hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
+                     (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+  constexpr size_t sm = dkv_smem<D, T>();
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
+    if (e != hipSuccess) return 2;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS>), dim3(nkt * p.Hkv * p.B), dim3(256), sm, s, p, (const T*)q, (const T*)k,
+                     (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
+  return 0;
+}
+
+template <typename T, int D, int KIND>
+static int launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                     const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
+  if (p.flags & FLEX_ROUND_S) return launch_one<T, D, KIND, true>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+  return launch_one<T, D, KIND, false>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+}
+
+template <typename T, int D>
+static int launch_kind(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
+  switch (p.score.kind) {
+    case FLEX_SCORE_IDENTITY: return launch_rs<T, D, FLEX_SCORE_IDENTITY>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+    case FLEX_SCORE_CHECKERBOARD: return launch_rs<T, D, FLEX_SCORE_CHECKERBOARD>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+    case FLEX_SCORE_ALIBI: return launch_rs<T, D, FLEX_SCORE_ALIBI>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+    case FLEX_SCORE_TANH_SOFTCAP: return launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+    case FLEX_SCORE_REL_BIAS: return launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+  }
+  return 1;
+}
+
+}  // namespace flex
+
+using namespace flex;
 void flex_set_error(const char* fmt, ...);
-bool flex_mfma_bwd_supported(const FlexAttnParams& p) { return false; }
-size_t flex_mfma_bwd_workspace(const FlexAttnParams& p) { return 0; }
+bool flex_mfma_shape_ok(const FlexAttnParams& p);
+
+bool flex_mfma_bwd_supported(const FlexAttnParams& p) {
+  if (!flex_mfma_shape_ok(p)) return false;
+  // the dK/dV kernel needs the transposed lists whenever lists are given
+  const FlexTileLists& t = p.tiles;
+  if (t.kv_num && (!t.q_num || !t.q_idx || !t.full_q_num || !t.full_q_idx)) return false;
+  return true;
+}
+
+size_t flex_mfma_bwd_workspace(const FlexAttnParams& p) { return 0; }  // delta is accounted for by the caller
+
 int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                  const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s) { flex_set_error("mfma bwd not built"); return 3; }
+                  const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s) {
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o | (uintptr_t)d_o | (uintptr_t)dq | (uintptr_t)dk | (uintptr_t)dv) & 15) {
+    flex_set_error("fused backward needs 16-byte aligned tensors");
+    return 1;
+  }
+  float* delta = (float*)workspace;
+  int rc;
+  if (p.dtype == FLEX_F16) rc = p.D == 64 ? launch_kind<f16, 64>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s)
+                                          : launch_kind<f16, 128>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+  else rc = p.D == 64 ? launch_kind<bf16, 64>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s)
+                      : launch_kind<bf16, 128>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+  if (rc == 1) flex_set_error("fused backward: unsupported score_mod kind %d", p.score.kind);
+  if (rc == 2) flex_set_error("fused backward: could not raise the dynamic LDS limit");
+  return rc;
+}

@@ -77,6 +77,7 @@ template <> struct Score2<FLEX_SCORE_IDENTITY> {
   float c;
   __device__ __forceinline__ void init(const FlexScoreMod&, float scale, int h) { c = scale * kLog2e; }
   __device__ __forceinline__ void tile(int q, int kvb) {}
+  __device__ __forceinline__ void tileT(int qb, int kv) {}
   __device__ __forceinline__ float apply(float s, int off) const { return s * c; }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
@@ -93,29 +94,37 @@ template <> struct Score2<FLEX_SCORE_CHECKERBOARD> {
     ce = par ? c1 : c0; co = par ? c0 : c1;
     fe = par ? f1 : f0; fo = par ? f0 : f1;
   }
+  // off runs along the query index instead (q = qb + off, fixed kv)
+  __device__ __forceinline__ void tileT(int qb, int kv) {
+    int par = (by_kv ? kv : (kv - qb)) & 1;
+    ce = par ? c1 : c0; fe = par ? f1 : f0;
+    if (by_kv) { co = ce; fo = fe; } else { co = par ? c0 : c1; fo = par ? f0 : f1; }
+  }
   __device__ __forceinline__ float apply(float s, int off) const { return s * ((off & 1) ? co : ce); }
   __device__ __forceinline__ float grad(float s, int off) const { return (off & 1) ? fo : fe; }
 };
 
 template <> struct Score2<FLEX_SCORE_ALIBI> {
-  float c, slope2, base;
+  float c, slope2, base, step;
   __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
     c = scale * kLog2e;
     slope2 = m.p0 * exp2f(-((float)(h + 1) * 8.0f / (float)m.i0)) * kLog2e;
   }
-  __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(q - kvb) * slope2; }
-  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, -slope2, base)); }
+  __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(q - kvb) * slope2; step = -slope2; }
+  __device__ __forceinline__ void tileT(int qb, int kv) { base = (float)(qb - kv) * slope2; step = slope2; }
+  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, step, base)); }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
 template <> struct Score2<FLEX_SCORE_REL_BIAS> {
-  float c, slope2, base;
+  float c, slope2, base, step;
   __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
     c = scale * kLog2e;
     slope2 = m.p0 * kLog2e;
   }
-  __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(kvb - q) * slope2; }
-  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, slope2, base)); }
+  __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(kvb - q) * slope2; step = slope2; }
+  __device__ __forceinline__ void tileT(int qb, int kv) { base = (float)(kv - qb) * slope2; step = -slope2; }
+  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, step, base)); }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
@@ -125,6 +134,7 @@ template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
     a = 2.f * kLog2e * scale * m.p1; cap2 = m.p0 * kLog2e; sc = scale;
   }
   __device__ __forceinline__ void tile(int q, int kvb) {}
+  __device__ __forceinline__ void tileT(int qb, int kv) {}
   __device__ __forceinline__ float tanh_(float s) const {
     float t = fast_exp2(fminf(s * a, 60.f));
     return 1.f - 2.f * fast_rcp(t + 1.f);
