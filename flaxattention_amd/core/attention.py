@@ -134,7 +134,8 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
         flags |= _lib.FLAG_ROUND_S
     if opts.get("backend", "auto") == "generic":
         flags |= _lib.FLAG_FORCE_GENERIC
-    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, opts.get("decode_splits", 0))
+    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True,
+                 opts.get("decode_splits", 0) if opts.get("decode", True) else 0)
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
         qb, kvb = _lib.C.c_int32(0), _lib.C.c_int32(0)

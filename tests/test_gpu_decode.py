@@ -1,0 +1,68 @@
+"""Split-KV decode kernel vs the CPU oracle, and vs the prefill kernel."""
+import pytest
+import torch
+
+import flaxattention_amd as fa
+from flaxattention_amd.masks import generate_sliding_window, offset_causal_mask
+from flaxattention_amd.mods import generate_alibi_bias, generate_tanh_softcap
+from oracle import (max_abs, o_alibi_config, o_offset_causal, o_tanh_softcap, ref_attention, rel_l2, seeded_qkv)
+
+pytestmark = pytest.mark.gpu
+
+
+def run_decode(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, splits, score=None, oscore=None, mask=None, omask=None):
+    print(f"decode case {dtype} B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv} D{D} splits{splits}", flush=True)
+    q, k, v = seeded_qkv(B, Hq, Hkv, Lq, Lkv, D, dtype)
+    bm = fa.create_block_mask(mask, B, Hq, Lq, Lkv, device=dev) if mask is not None else None
+    out, lse = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=score, block_mask=bm,
+                                 enable_gqa=Hq != Hkv, return_lse=True, kernel_options={"decode_splits": splits})
+    want, want_lse = ref_attention(q, k, v, oscore, omask, strict=True, return_lse=True)
+    a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
+    print(f"  O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
+    assert a <= 2e-2 and r <= (1e-3 if dtype == torch.float16 else 6e-3)
+    dead = torch.isneginf(want_lse)
+    assert torch.equal(torch.isneginf(lse.cpu()), dead)
+    assert max_abs(lse.cpu()[~dead], want_lse[~dead]) <= 2e-2
+    return out
+
+
+@pytest.mark.parametrize("Lq", [1, 16, 64])
+@pytest.mark.parametrize("splits", [1, 5, 16])
+def test_decode_alibi_offset_causal(dev, Lq, splits):
+    # benchmark configuration 5 at reduced KV length
+    Lkv = 2048
+    run_decode(dev, torch.float16, 2, 8, 8, Lq, Lkv, 64, splits, generate_alibi_bias(8, -1.0), o_alibi_config(8),
+               offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq))
+
+
+def test_decode_gqa_packs_heads(dev):
+    run_decode(dev, torch.bfloat16, 2, 8, 2, 4, 1000, 128, 4, generate_tanh_softcap(30.0), o_tanh_softcap(30.0),
+               offset_causal_mask(996), o_offset_causal(996))
+    run_decode(dev, torch.float16, 1, 16, 2, 8, 777, 64, 3)       # 64 columns, no mask, ragged KV
+
+
+def test_decode_window_uses_tile_lists(dev):
+    # only the last 300 keys are visible: most tiles are skipped through the lists
+    Lkv, Lq, W = 4096, 2, 300
+    from oracle import o_and_masks
+    def owin(b, h, q_idx, kv_idx):
+        return (q_idx + (Lkv - Lq) - kv_idx <= W) & (q_idx + (Lkv - Lq) >= kv_idx)
+    from flaxattention_amd.core.common import MaskMod
+    mask = MaskMod(lo=0, hi=W, sink=-1, q_offset=Lkv - Lq, name="decode_window")
+    run_decode(dev, torch.float16, 1, 4, 4, Lq, Lkv, 64, 8, mask=mask, omask=owin)
+
+
+def test_decode_independent_of_split_count(dev):
+    q, k, v = (t.to(dev) for t in seeded_qkv(1, 4, 4, 1, 4096, 64, torch.float16))
+    outs = [fa.flax_attention(q, k, v, kernel_options={"decode_splits": s}) for s in (1, 2, 7, 32)]
+    for o in outs[1:]:
+        assert max_abs(o.cpu(), outs[0].cpu()) <= 2e-3
+
+
+def test_decode_matches_prefill_kernel(dev):
+    q, k, v = (t.to(dev) for t in seeded_qkv(2, 8, 8, 16, 4096, 64, torch.float16))
+    m = offset_causal_mask(4096 - 16)
+    bm = fa.create_block_mask(m, 1, 1, 16, 4096, device=dev)
+    a = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(8, -1.0), block_mask=bm, kernel_options={"decode_splits": 16})
+    b = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(8, -1.0), block_mask=bm, kernel_options={"decode_splits": 0, "decode": False})
+    assert max_abs(a.cpu(), b.cpu()) <= 4e-3
