@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the FlexAttention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config2|config3|config4|config5]
+                    [--no-cpu] [--all]
+
+A "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM.  The default workload is benchmark configuration 2
+(fp16 [8,8,2048,64], checkerboard score_mod, no mask, forward + backward of
+out.sum()); one step = forward kernel + both backward kernels.  The last line
+printed on stdout is ONE JSON object (the driver's contract); --all prints
+per-configuration lines to stderr first.
+
+Throughput counts algorithmic flops only: 4*bq*bk*D per visible tile in the
+forward and 10*bq*bk*D in the backward at the 128x128 granularity of the block
+mask, recomputation in the split backward kernels not counted.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
+PEAK_HBM_GBPS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class Prepared:
+    """One problem with every buffer and the C parameter block prepared once,
+    so that the timed loop is nothing but C-ABI calls on torch's current stream."""
+
+    def __init__(self, dev, dtype, B, Hq, Hkv, Lq, Lkv, D, score, mask, opts=None, seed=0, decode_splits=0):
+        import flaxattention_amd as fa
+        from flaxattention_amd import _lib
+        from flaxattention_amd.core.attention import _make_plan
+        self.L = _lib.lib()
+        self._lib = _lib
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(dtype).to(dev)
+        self.k, self.q, self.v = mk(B, Hkv, Lkv, D), mk(B, Hq, Lq, D), mk(B, Hkv, Lkv, D)
+        self.d_o = torch.ones(B, Hq, Lq, D, dtype=dtype, device=dev)   # gradient of out.sum()
+        bm = fa.create_block_mask(mask, 1, 1, Lq, Lkv, device=dev) if mask is not None else None
+        self.block_mask = bm
+        opts = dict(opts or {})
+        if decode_splits:
+            opts["decode_splits"] = decode_splits
+        self.plan = _make_plan(self.q, self.k, self.v, score, bm, None, 1.0 / D ** 0.5, opts)
+        self.o = torch.empty(B, Hq, Lq, D, dtype=dtype, device=dev)
+        self.lse = torch.empty(B, Hq, Lq, dtype=torch.float32, device=dev)
+        self.dq, self.dk, self.dv = torch.empty_like(self.q), torch.empty_like(self.k), torch.empty_like(self.v)
+        self.p = self.plan.params(self.q, self.k, self.v, self.o)
+        self.ws = torch.empty(max(self.L.flexattn_bwd_workspace_bytes(self.p), 256), dtype=torch.uint8, device=dev)
+        self.splits = decode_splits
+        if decode_splits:
+            n = self.L.flexattn_decode_workspace_bytes(self.p, decode_splits)
+            self.dws = torch.empty(max(n, 256), dtype=torch.uint8, device=dev)
+        self.stream = torch.cuda.current_stream(dev).cuda_stream
+        self.ptr = {n: getattr(self, n).data_ptr() for n in ("q", "k", "v", "o", "lse", "d_o", "dq", "dk", "dv", "ws")}
+        self.p_dq = self._with_flags(_lib.FLAG_BWD_ONLY_DQ)
+        self.p_dkv = self._with_flags(_lib.FLAG_BWD_ONLY_DKV)
+
+    def _with_flags(self, extra):
+        p2 = self._lib.FlexAttnParams()
+        C.memmove(C.byref(p2), C.byref(self.p), C.sizeof(self.p))
+        p2.flags = self.p.flags | extra
+        return p2
+
+    def fwd(self):
+        t = self.ptr
+        rc = self.L.flexattn_fwd(self.p, t["q"], t["k"], t["v"], t["o"], t["lse"], None, self.stream)
+        if rc:
+            self._lib.check(rc, "flexattn_fwd")
+
+    def decode(self):
+        t = self.ptr
+        rc = self.L.flexattn_decode(self.p, t["q"], t["k"], t["v"], t["o"], t["lse"], self.splits, self.dws.data_ptr(), self.stream)
+        if rc:
+            self._lib.check(rc, "flexattn_decode")
+
+    def bwd(self, which=None):
+        t = self.ptr
+        p = self.p if which is None else (self.p_dq if which == "dq" else self.p_dkv)
+        rc = self.L.flexattn_bwd(p, t["q"], t["k"], t["v"], t["o"], t["lse"], t["d_o"], t["dq"], t["dk"], t["dv"], t["ws"], self.stream)
+        if rc:
+            self._lib.check(rc, "flexattn_bwd")
+
+
+def event_time_us(fn, n, warm=3):
+    """Average duration of fn's launches, HIP events on the launch stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / n
+
+
+def wall_time_ms(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def tiles_128(mask_name, L):
+    n = L // 128
+    if mask_name == "none":
+        return n * n
+    if mask_name == "causal":
+        return n * (n + 1) // 2
+    raise ValueError(mask_name)
+
+
+def cpu_baseline(workload):
+    """The oracle (a CPU restatement of the reference's dense path) timed on
+    this host on a bounded slice of the same workload."""
+    from oracle import (o_alibi_config, o_causal_mask, o_checkerboard_kv, ref_attention, ref_attention_bwd, seeded_qkv)
+    torch.set_num_threads(os.cpu_count() or 1)
+    cores = torch.get_num_threads()
+    if workload == "config3":
+        dtype, sm, mm, flops, tag = torch.bfloat16, o_alibi_config(8), o_causal_mask, 127.78e9 / 8, "ALiBi + causal"
+    else:
+        dtype, sm, mm, flops, tag = torch.float16, o_checkerboard_kv, None, 240.52e9 / 8, "checkerboard"
+    q, k, v = seeded_qkv(1, 8, 8, 2048, 2048, 64, dtype)
+    d_o = torch.ones_like(q)
+    t0 = time.perf_counter()
+    ref_attention(q, k, v, sm, mm, strict=True)
+    ref_attention_bwd(q, k, v, d_o, sm, mm, strict=True)
+    dt = time.perf_counter() - t0
+    return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"1 of 8 batch elements of the workload ([1,8,2048,64] {str(dtype).split('.')[-1]}, {tag}), "
+                      f"forward + backward once, {dt:.1f} s"}
+
+
+def run_train_config(dev, name, steps, warmup, opts=None):
+    from flaxattention_amd.masks import causal_mask
+    from flaxattention_amd.mods import generate_alibi_bias, generate_checkerboard
+    if name == "config2":
+        # the configuration's spelling of the checkerboard: x0.5 where kv_idx is odd, x2.0 where even; no mask
+        pr = Prepared(dev, torch.float16, 8, 8, 8, 2048, 2048, 64, generate_checkerboard(2.0, 0.5, "kv"), None, opts)
+        tiles, dtype = 8 * 8 * tiles_128("none", 2048), "fp16"
+    else:
+        pr = Prepared(dev, torch.bfloat16, 8, 8, 8, 2048, 2048, 64, generate_alibi_bias(8, -1.0), causal_mask, opts)
+        tiles, dtype = 8 * 8 * tiles_128("causal", 2048), "bf16"
+    per_tile = 128 * 128 * 64
+    f_fwd, f_bwd = 4 * per_tile * tiles, 10 * per_tile * tiles
+
+    def step():
+        pr.fwd()
+        pr.bwd()
+    ms = wall_time_ms(step, steps, warmup)
+    n = max(steps, 10)
+    us = {"fwd_mfma_kernel": event_time_us(pr.fwd, n),
+          "bwd_dq_kernel": event_time_us(lambda: pr.bwd("dq"), n),
+          "bwd_dkv_kernel": event_time_us(lambda: pr.bwd("dkv"), n)}
+    alg = {"fwd_mfma_kernel": f_fwd, "bwd_dq_kernel": 2 * per_tile * tiles, "bwd_dkv_kernel": 8 * per_tile * tiles}
+    kern = {k: {"us": round(us[k], 2), "algorithmic_flops": alg[k], "tflops": round(alg[k] / us[k] / 1e6, 1)} for k in us}
+    dom = max(us, key=us.get)
+    return {"ms_per_step": ms, "tflops": (f_fwd + f_bwd) / ms / 1e9, "fwd_tflops": f_fwd / us["fwd_mfma_kernel"] / 1e6,
+            "bwd_tflops": f_bwd / (us["bwd_dq_kernel"] + us["bwd_dkv_kernel"]) / 1e6,
+            "kernels": kern, "dominant": dom, "dtype": dtype, "flops": f_fwd + f_bwd}
+
+
+def run_config4(dev, steps, warmup):
+    from flaxattention_amd.masks import generate_attention_sink
+    from flaxattention_amd.mods import generate_tanh_softcap
+    # |q-kv| <= 1024 causal window, kv < 4 always visible, tanh soft-cap 50
+    pr = Prepared(dev, torch.bfloat16, 4, 16, 16, 8192, 8192, 128, generate_tanh_softcap(50.0), generate_attention_sink(1024, 3))
+    bm = pr.block_mask
+    tiles = int(bm.kv_num_blocks.sum().item() + bm.full_kv_num_blocks.sum().item()) * 4 * 16
+    flops = 4 * 128 * 128 * 128 * tiles
+    us = event_time_us(pr.fwd, max(steps, 10))
+    return {"us": us, "tflops": flops / us / 1e6, "tiles_per_head": tiles // 64}
+
+
+def run_config5(dev, steps, warmup, sweep=True):
+    from flaxattention_amd.masks import offset_causal_mask
+    from flaxattention_amd.mods import generate_alibi_bias
+    out = {}
+    Lkv = 16384
+    for ql in (1, 16, 64):
+        byts = 2 * 8 * 8 * Lkv * 64 * 2 + 2 * 8 * 8 * ql * 64 * 2
+        best = None
+        for splits in ((8, 16) if sweep else (8,)):
+            pr = Prepared(dev, torch.float16, 8, 8, 8, ql, Lkv, 64, generate_alibi_bias(8, -1.0), offset_causal_mask(Lkv - ql),
+                          decode_splits=splits)
+            us = event_time_us(pr.decode, max(steps, 20))
+            if best is None or us < best[0]:
+                best = (us, splits)
+        pr = Prepared(dev, torch.float16, 8, 8, 8, ql, Lkv, 64, generate_alibi_bias(8, -1.0), offset_causal_mask(Lkv - ql))
+        us_pre = event_time_us(pr.fwd, max(steps, 10))
+        out[ql] = {"decode_us": best[0], "splits": best[1], "decode_gbps": byts / best[0] / 1e3,
+                   "prefill_kernel_us": us_pre, "bytes": byts}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--all", action="store_true", help="also run configurations 3, 4 and 5 (reported on stderr and in 'extra')")
+    ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (attention shards over batch x head "
+              "without communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda", 0)
+    opts = {"round_s": bool(a.round_s)}
+    r = run_train_config(dev, a.workload, a.steps, a.warmup, opts)
+    log(f"{a.workload}: {r['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r['tflops']:.1f} TFLOP/s  "
+        f"(fwd {r['fwd_tflops']:.1f}, bwd {r['bwd_tflops']:.1f})  kernels {r['kernels']}")
+    extra = {}
+    if a.all:
+        other = "config3" if a.workload == "config2" else "config2"
+        r2 = run_train_config(dev, other, a.steps, a.warmup, opts)
+        log(f"{other}: {r2['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r2['tflops']:.1f} TFLOP/s  kernels {r2['kernels']}")
+        extra[other] = {"ms_per_step": round(r2["ms_per_step"], 4), "fwd_bwd_tflops": round(r2["tflops"], 1), "kernels": r2["kernels"]}
+        c4 = run_config4(dev, a.steps, a.warmup)
+        log(f"config4: fwd {c4['us']:.1f} us  {c4['tflops']:.1f} TFLOP/s on {c4['tiles_per_head']} tiles/head")
+        extra["config4"] = {"fwd_us": round(c4["us"], 1), "fwd_tflops": round(c4["tflops"], 1)}
+        c5 = run_config5(dev, a.steps, a.warmup)
+        for ql, d in c5.items():
+            log(f"config5 q_len {ql}: decode {d['decode_us']:.1f} us ({d['decode_gbps']:.0f} GB/s, {d['decode_gbps'] / PEAK_HBM_GBPS * 100:.1f}% of HBM peak, "
+                f"{d['splits']} splits); prefill kernel {d['prefill_kernel_us']:.1f} us")
+        extra["config5"] = {str(ql): {"decode_us": round(d["decode_us"], 1), "decode_gbps": round(d["decode_gbps"]),
+                                      "frac_hbm_peak": round(d["decode_gbps"] / PEAK_HBM_GBPS, 3), "splits": d["splits"],
+                                      "prefill_kernel_us": round(d["prefill_kernel_us"], 1)} for ql, d in c5.items()}
+    dom = r["dominant"]
+    kd = r["kernels"][dom]
+    line = {
+        "metric": "fwd+bwd TFLOP/s (B8 H8 L2048 D64, algorithmic flops of unmasked 128x128 tiles)",
+        "value": round(r["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(r["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": r["dtype"], "data": "synthetic",
+        "config": {"workload": {"config2": "configs[1]: fp16 [8,8,2048,64] checkerboard score_mod, no mask, forward + backward of out.sum()",
+                                "config3": "configs[2]: bf16 [8,8,2048,64] ALiBi score_mod, causal block mask 128x128, forward + backward of out.sum()"}[a.workload],
+                   "round_s": bool(a.round_s)},
+        "pct_mfma_peak": round(r["tflops"] / PEAK_MFMA_TFLOPS * 100, 2),
+        "fwd_tflops": round(r["fwd_tflops"], 1), "bwd_tflops": round(r["bwd_tflops"], 1),
+        "kernels": r["kernels"],
+        "roofline": {"bound": "mfma", "kernel": dom, "achieved": kd["tflops"], "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(kd["tflops"] / PEAK_MFMA_TFLOPS, 4), "traffic": None},
+    }
+    if extra:
+        line["extra"] = extra
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.workload)
+        log(f"cpu baseline: {line['cpu_baseline']}")
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -70,7 +70,12 @@ enum FlexFlags {
   FLEX_STRICT = 2,       /* generic kernels only: also round the normalised P,
                             dP and dS through the input dtype (attention.py:105
                             and its transposes) */
-  FLEX_FORCE_GENERIC = 4 /* never use the MFMA kernels */
+  FLEX_FORCE_GENERIC = 4, /* never use the MFMA kernels */
+  /* profiling aids for flexattn_bwd: launch only one of the two fused backward
+   * kernels.  The dK/dV kernel then reads the delta values a previous complete
+   * call left in the same workspace. */
+  FLEX_BWD_ONLY_DQ = 8,
+  FLEX_BWD_ONLY_DKV = 16
 };
 
 /* Ordered tile lists in the layout of BlockMask.kv_num_blocks / kv_indices /
