@@ -1,0 +1,206 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports every
+symbol the header declares, ctypes structs match the C layout, mask / score
+functors fold and evaluate like the oracle's restatements, Python callables
+are recognised, and argument validation raises the reference's errors."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import flaxattention_amd as fa
+from flaxattention_amd import _lib
+from flaxattention_amd.core.common import (INT_MAX, INT_MIN, MaskMod, ScoreMod, _fit_band, _get_mod_type,
+                                           _ModificationType, _probe_score_mod, pack_bits, resolve_score_mod)
+from flaxattention_amd.masks import (causal_mask, generate_attention_sink, generate_sliding_window, offset_causal_mask)
+from flaxattention_amd.mods import (checkerboard, generate_alibi_bias, generate_checkerboard, generate_rel_bias,
+                                    generate_tanh_softcap)
+from oracle import (o_alibi, o_alibi_config, o_attention_sink, o_causal_mask, o_checkerboard, o_checkerboard_kv,
+                    o_noop_mask, o_offset_causal, o_rel_bias, o_sink_window_lt, o_sliding_window, o_tanh_softcap)
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flexattn.h")
+
+
+def test_library_exports_every_declared_symbol():
+    decl = set(re.findall(r"\b(flexattn_[a-z_]+)\s*\(", open(HEADER).read()))
+    assert decl == set(_lib.EXPORTS), decl ^ set(_lib.EXPORTS)
+    L = _lib.lib()
+    for name in decl:
+        assert hasattr(L, name), name
+    assert L.flexattn_abi_version() == 1
+    assert L.flexattn_last_error() is not None
+
+
+def test_ctypes_structs_match_c_layout(tmp_path):
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "flexattn.h"\n'
+                   'int main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(FlexScoreMod), sizeof(FlexMask),'
+                   'sizeof(FlexTileLists), sizeof(FlexAttnParams), offsetof(FlexAttnParams, scale),'
+                   'offsetof(FlexAttnParams, score), offsetof(FlexAttnParams, mask), offsetof(FlexAttnParams, tiles));return 0;}\n')
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    got = [int(x) for x in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
+    P = _lib.FlexAttnParams
+    want = [ctypes.sizeof(_lib.FlexScoreMod), ctypes.sizeof(_lib.FlexMask), ctypes.sizeof(_lib.FlexTileLists),
+            ctypes.sizeof(P), P.scale.offset, P.score.offset, P.mask.offset, P.tiles.offset]
+    assert got == want
+
+
+def test_workspace_and_tile_queries_without_gpu():
+    L = _lib.lib()
+    assert L.flexattn_block_mask_workspace_bytes(2, 3, 4, 5) >= 2 * 2 * 3 * 4 * 5
+    qb, kvb = ctypes.c_int32(), ctypes.c_int32()
+    L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (128, 64)
+    L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (0, 0)
+    # argument validation happens before anything touches a device
+    p = _lib.FlexAttnParams()
+    assert L.flexattn_fwd(p, None, None, None, None, None, None, None) != 0
+    assert b"flexattn_fwd" in L.flexattn_last_error()
+
+
+GRID = dict(b=torch.arange(2, dtype=torch.int32).reshape(2, 1, 1, 1), h=torch.arange(4, dtype=torch.int32).reshape(1, 4, 1, 1),
+            q=torch.arange(70, dtype=torch.int32).reshape(1, 1, 70, 1), kv=torch.arange(90, dtype=torch.int32).reshape(1, 1, 1, 90))
+
+
+def same_mask(a, b):
+    x = torch.broadcast_to(torch.as_tensor(a(GRID["b"], GRID["h"], GRID["q"], GRID["kv"])), (2, 4, 70, 90))
+    y = torch.broadcast_to(torch.as_tensor(b(GRID["b"], GRID["h"], GRID["q"], GRID["kv"])), (2, 4, 70, 90))
+    return torch.equal(x.bool(), y.bool())
+
+
+def test_mask_functors_match_reference_definitions():
+    assert same_mask(causal_mask, o_causal_mask)                               # masks/causal.py:4-5
+    assert same_mask(generate_sliding_window(10), o_sliding_window(10))        # masks/sliding_window.py:7-22
+    assert same_mask(generate_attention_sink(20, 4), o_attention_sink(20, 4))  # masks/attention_sink.py:6-24
+    assert same_mask(generate_attention_sink(20, 3), o_sink_window_lt(20, 4))
+    assert same_mask(offset_causal_mask(30), o_offset_causal(30))
+    assert same_mask(fa.noop_mask, o_noop_mask)
+    assert generate_sliding_window(10).__name__ == "sliding_window_10"
+    assert generate_attention_sink(32, 4).__name__ == "attention_sink_32_4"
+
+
+def test_and_or_masks_fold_and_fall_back():
+    m = fa.and_masks(causal_mask, generate_sliding_window(10))                 # examples/example.py:40
+    assert isinstance(m, MaskMod) and (m.lo, m.hi, m.sink) == (0, 10, -1)
+    sink = generate_attention_sink(1024, 4)
+    assert (sink.lo, sink.hi, sink.sink) == (0, 1024, 4)
+    u = fa.or_masks(causal_mask, generate_sliding_window(5))
+    assert same_mask(u, o_causal_mask)
+
+    def odd_rows(b, h, q_idx, kv_idx):
+        return q_idx % 2 == 1
+    mixed = fa.and_masks(causal_mask, odd_rows)
+    assert not isinstance(mixed, MaskMod)
+    assert same_mask(mixed, lambda b, h, q, kv: (q >= kv) & (q % 2 == 1))
+    with pytest.raises(RuntimeError):
+        fa.or_masks(causal_mask, "nope")
+    with pytest.raises(RuntimeError):
+        fa.and_masks(1, causal_mask)
+    assert same_mask(fa.and_masks(), o_noop_mask)
+    assert not torch.as_tensor(fa.or_masks()(0, 0, torch.arange(3), torch.arange(3))).any()
+
+
+def test_band_fit_and_bit_packing():
+    q, kv = torch.arange(256).reshape(-1, 1), torch.arange(384).reshape(1, -1)
+    for lo, hi, sink in ((0, INT_MAX, -1), (0, 40, -1), (0, 40, 3), (-7, 9, -1), (INT_MIN, INT_MAX, -1)):
+        d = q - kv
+        m = (d >= lo) & ((d <= hi) | (kv <= sink))
+        f = _fit_band(m)
+        assert f is not None
+        assert torch.equal((d >= f.lo) & ((d <= f.hi) | (kv <= f.sink)), m)
+    assert _fit_band((q * 7 + kv) % 5 < 2) is None
+    allf = _fit_band(torch.zeros(128, 128, dtype=torch.bool))
+    assert allf.lo == INT_MAX
+    m = torch.rand(2, 3, 17, 70, generator=torch.Generator().manual_seed(1)) < 0.5
+    w = pack_bits(m)
+    assert w.shape == (2, 3, 17, 3) and w.dtype == torch.int32
+    for kvx in (0, 31, 32, 69):
+        assert torch.equal(((w[..., kvx >> 5] >> (kvx & 31)) & 1).bool(), m[..., kvx])
+
+
+SGRID = dict(s=torch.linspace(-3, 3, 5).reshape(5, 1, 1, 1, 1), b=torch.zeros(1, 1, 1, 1, 1, dtype=torch.int32),
+             h=torch.arange(8, dtype=torch.int32).reshape(1, 1, 8, 1, 1), q=torch.arange(9, dtype=torch.int32).reshape(1, 1, 1, 9, 1),
+             kv=torch.arange(11, dtype=torch.int32).reshape(1, 1, 1, 1, 11))
+
+
+def same_score(a, b):
+    sh = (5, 1, 8, 9, 11)
+    x = torch.broadcast_to(a(SGRID["s"].expand(sh), SGRID["b"], SGRID["h"], SGRID["q"], SGRID["kv"]), sh)
+    y = torch.broadcast_to(b(SGRID["s"].expand(sh), SGRID["b"], SGRID["h"], SGRID["q"], SGRID["kv"]), sh)
+    return torch.allclose(x, y, rtol=1e-6, atol=1e-6)
+
+
+def test_score_functors_match_reference_definitions():
+    assert same_score(generate_alibi_bias(8), o_alibi(8))                       # mods/alibi.py:15-18
+    assert same_score(generate_alibi_bias(8, -1.0), o_alibi_config(8))
+    assert same_score(checkerboard, o_checkerboard)                             # examples/benchmark.py:16-22
+    assert same_score(generate_checkerboard(2.0, 0.5, "kv"), o_checkerboard_kv)
+    assert same_score(generate_tanh_softcap(50.0), o_tanh_softcap(50.0))
+    assert same_score(generate_rel_bias(0.1), o_rel_bias(0.1))
+
+
+def test_untagged_score_mods_are_recognised():
+    def my_alibi(score, b, h, q_idx, kv_idx):
+        return score + (q_idx - kv_idx) * torch.exp2(-((h + 1) * 8.0 / 8))
+    s = resolve_score_mod(my_alibi, 8)
+    assert (s.kind, s.p0, s.i0) == (_lib.SCORE_ALIBI, 1.0, 8)
+    assert resolve_score_mod(o_checkerboard, 4).key() == (_lib.SCORE_CHECKERBOARD, 0.5, 2.0, 0)
+    assert resolve_score_mod(o_checkerboard_kv, 4).key() == (_lib.SCORE_CHECKERBOARD, 2.0, 0.5, 1)
+    c = resolve_score_mod(o_tanh_softcap(30.0), 4)
+    assert c.kind == _lib.SCORE_TANH_SOFTCAP and abs(c.p0 - 30.0) < 1e-4
+    r = resolve_score_mod(o_rel_bias(-0.25), 4)
+    assert r.kind == _lib.SCORE_REL_BIAS and abs(r.p0 + 0.25) < 1e-6
+    assert resolve_score_mod(lambda s, b, h, q, kv: s, 4).kind == _lib.SCORE_IDENTITY
+    assert resolve_score_mod(None, 4).kind == _lib.SCORE_IDENTITY
+    assert _probe_score_mod(lambda s, b, h, q, kv: s * s, 4) is None
+    with pytest.raises(NotImplementedError):
+        resolve_score_mod(lambda s, b, h, q, kv: torch.sin(s), 4)
+
+
+def test_mod_type_by_arity():
+    assert _get_mod_type(lambda b, h, q, kv: True) == _ModificationType.MASK_MOD
+    assert _get_mod_type(lambda s, b, h, q, kv: s) == _ModificationType.SCORE_MOD
+    assert _get_mod_type(causal_mask) == _ModificationType.MASK_MOD
+    assert _get_mod_type(checkerboard) == _ModificationType.SCORE_MOD
+    with pytest.raises(AssertionError):
+        _get_mod_type(lambda a, b: a)
+
+
+def test_front_end_validation_raises_reference_errors():
+    q, k, v = torch.zeros(1, 4, 8, 16), torch.zeros(1, 2, 8, 16), torch.zeros(1, 2, 8, 16)
+    with pytest.raises(ValueError, match="same number of heads"):
+        fa.flax_attention(q, k, v)
+    with pytest.raises(ValueError, match="same dtype"):
+        fa.flax_attention(q, k.half(), v)
+    with pytest.raises(NotImplementedError, match="4D"):
+        fa.flax_attention(q[0], k[0], v[0], enable_gqa=True)
+    with pytest.raises(ValueError, match="embedding dimension"):
+        fa.flax_attention(q, k[..., :8], v, enable_gqa=True)
+    with pytest.raises(ValueError, match="value embedding dimension"):
+        fa.flax_attention(q, k, torch.zeros(1, 2, 8, 32), enable_gqa=True)
+    with pytest.raises(ValueError, match="multiple of kv heads"):
+        fa.flax_attention(torch.zeros(1, 3, 8, 16), k, v, enable_gqa=True)
+    with pytest.raises(ValueError, match="same number of heads"):
+        fa.flax_attention_pallas(q, k, v)
+    # valid arguments on the CPU: there is no fallback, the call must fail loudly
+    with pytest.raises(fa.FlexAttnError, match="no CPU fallback"):
+        fa.flax_attention(q, k, v, enable_gqa=True)
+    with pytest.raises(ValueError, match="only one of"):
+        fa.flax_attention_pallas(q, k, v, mask_mod=causal_mask, block_mod=causal_mask, enable_gqa=True)
+
+
+def test_product_never_imports_the_oracle():
+    code = "import sys; import flaxattention_amd, flaxattention_amd.masks, flaxattention_amd.mods; " \
+           "assert not any(m == 'oracle' or m.startswith('oracle.') for m in sys.modules), 'oracle imported'"
+    subprocess.run([sys.executable, "-c", code], check=True, cwd=ROOT)
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "flaxattention_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cuh")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f
