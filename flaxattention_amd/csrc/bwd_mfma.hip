@@ -39,9 +39,9 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
   const int nqt = (p.Lq + BM - 1) / BM;
   const int total = nqt * p.Hq * p.B;
-  const int wid = xcd_remap(blockIdx.x, total);
-  const int qt = nqt - 1 - (wid % nqt);
-  const int bh = wid / nqt;
+  int rank, bh;
+  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
+  const int qt = nqt - 1 - rank;
   const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
   const int q_row = qt * BM + w * 32 + i32;
   const int q_ld = min(q_row, p.Lq - 1);
@@ -122,13 +122,17 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
 #pragma unroll
     for (int r = 0; r < 16; r++) dqacc[db][r] = 0.f;
 
-  if (nt > 0) load_tile(tile_at(0) * BN);
+  int t_cur = nt > 0 ? tile_at(0) : 0;
+  int t_nxt = nt > 1 ? tile_at(1) : 0;
+  if (nt > 0) load_tile(t_cur * BN);
   for (int it = 0; it < nt; it++) {
-    const int kv0 = tile_at(it) * BN;
+    const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
     store_tile();
     __syncthreads();
-    if (it + 1 < nt) load_tile(tile_at(it + 1) * BN);
+    if (it + 1 < nt) load_tile(t_nxt * BN);
+    t_cur = t_nxt;
+    if (it + 2 < nt) t_nxt = tile_at(it + 2);
 
     float16_t sacc[2], dpacc[2];
 #pragma unroll
@@ -143,22 +147,40 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
         dpacc[nb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + 16 * s), dof[s], dpacc[nb]);
       }
     }
-    vec8 dsf[4];
+    // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
+    float16_t gacc[2];
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
-      const int kvb = kv0 + nb * 32 + 4 * g;
-      sm.tile(q_row, kvb);
+      sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float s = sacc[nb][r];
-        if (ROUND_S) s = round_through<T>(s);
-        float x = sm.apply(s, acc_row(r));
-        if (masked) x = visible(q_row, kvb + acc_row(r)) ? x : -INFINITY;
-        float pr = fast_exp2(x - lse);
-        float ds = pr * (dpacc[nb][r] - delta) * (sm.grad(s, acc_row(r)) * p.scale);
-        dsf[2 * nb + r / 8][r % 8] = (T)ds;
+      for (int r = 0; r < 16; r += 2) {
+        float s0 = sacc[nb][r], s1 = sacc[nb][r + 1];
+        if (ROUND_S) round_pair<T>(s0, s1);
+        sacc[nb][r] = sm.apply_sub(s0, acc_row(r), lse);
+        sacc[nb][r + 1] = sm.apply_sub(s1, acc_row(r + 1), lse);
+        if (!Score2<KIND>::kGradOne) {
+          gacc[nb][r] = sm.grad(s0, acc_row(r));
+          gacc[nb][r + 1] = sm.grad(s1, acc_row(r + 1));
+        }
       }
     }
+    if (masked) mask_tile_q(sacc, p.mask, visible, q_row, kv0, g, p.Lkv);
+    vec8 dsf[4];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++)
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++) {
+        typename Pair<T>::v2 pr[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const int r = 8 * tt + 2 * e;
+          float d0 = fast_exp2(sacc[nb][r]) * (dpacc[nb][r] - delta);
+          float d1 = fast_exp2(sacc[nb][r + 1]) * (dpacc[nb][r + 1] - delta);
+          if (!Score2<KIND>::kGradOne) { d0 *= gacc[nb][r]; d1 *= gacc[nb][r + 1]; }
+          pr[e] = Pair<T>::pack(d0, d1);
+        }
+        dsf[2 * nb + tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+      }
 #pragma unroll
     for (int t = 0; t < 4; t++) {
 #pragma unroll
@@ -172,6 +194,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
     __syncthreads();
   }
 
+  // the scale factor of dS = P o (dP - delta) o g * scale is applied once here
   if (q_row < p.Lq) {
     T* op = dq + row_id * D + 4 * g;
 #pragma unroll
@@ -180,7 +203,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
       for (int rr = 0; rr < 4; rr++) {
         union { T e[4]; uint2 u; } pk;
 #pragma unroll
-        for (int e = 0; e < 4; e++) pk.e[e] = (T)dqacc[db][4 * rr + e];
+        for (int e = 0; e < 4; e++) pk.e[e] = (T)(dqacc[db][4 * rr + e] * p.scale);
         *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
       }
   }
@@ -208,9 +231,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
   const int wk = w & 1, wq = w >> 1;
   const int nkt = (p.Lkv + BN - 1) / BN;
   const int total = nkt * p.Hkv * p.B;
-  const int wid = xcd_remap(blockIdx.x, total);
-  const int kt = wid % nkt;  // early key tiles see the most queries under causal masks
-  const int bh = wid / nkt;
+  int kt, bh;  // early key tiles see the most queries under causal masks
+  xcd_tile_map(blockIdx.x, nkt, p.Hkv * p.B, kt, bh);
   const int hk = bh % p.Hkv, b = bh / p.Hkv, G = p.Hq / p.Hkv;
   const int kv_col = kt * BN + wk * 32 + i32;
   const int kv_ld = min(kv_col, p.Lkv - 1);
@@ -255,33 +277,52 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
     const int64_t rows0 = ((int64_t)b * p.Hq + h) * p.Lq;
     const T* dobase = d_o + rows0 * D;
 
+    auto tile_at = [&](int it) -> int {
+      if (!full_idx) return it;
+      return it < n_full ? full_idx[it] : part_idx[it - n_full];
+    };
+    uint4 qreg[NLD], oreg[NLD];
+    float lreg = INFINITY, dreg = 0.f;
+    auto load_tile = [&](int q0) {
+#pragma unroll
+      for (int j = 0; j < NLD; j++) {
+        int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+        qreg[j] = make_uint4(0, 0, 0, 0);
+        oreg[j] = make_uint4(0, 0, 0, 0);
+        if (q0 + r < p.Lq) {
+          qreg[j] = *reinterpret_cast<const uint4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
+          oreg[j] = *reinterpret_cast<const uint4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
+        }
+      }
+      lreg = INFINITY;
+      dreg = 0.f;
+      if (tid < BM && q0 + tid < p.Lq) {
+        lreg = lse2[rows0 + q0 + tid];
+        dreg = delta[rows0 + q0 + tid];
+        if (lreg == -INFINITY) lreg = INFINITY;  // row without visible keys: P = 0
+      }
+    };
+    int t_cur = nt > 0 ? tile_at(0) : 0;
+    int t_nxt = nt > 1 ? tile_at(1) : 0;
+    if (nt > 0) load_tile(t_cur * BM);
     for (int it = 0; it < nt; it++) {
-      const int qtile = full_idx ? (it < n_full ? full_idx[it] : part_idx[it - n_full]) : it;
-      const int q0 = qtile * BM;
+      const int q0 = t_cur * BM;
       const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
       __syncthreads();  // previous tile fully consumed
 #pragma unroll
       for (int j = 0; j < NLD; j++) {
         int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-        uint4 a = make_uint4(0, 0, 0, 0), d4 = make_uint4(0, 0, 0, 0);
-        if (q0 + r < p.Lq) {
-          a = *reinterpret_cast<const uint4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
-          d4 = *reinterpret_cast<const uint4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
-        }
-        *reinterpret_cast<uint4*>(Qs + r * ROWE + cc * 8) = a;
-        *reinterpret_cast<uint4*>(Os + r * ROWE + cc * 8) = d4;
+        *reinterpret_cast<uint4*>(Qs + r * ROWE + cc * 8) = qreg[j];
+        *reinterpret_cast<uint4*>(Os + r * ROWE + cc * 8) = oreg[j];
       }
       if (tid < BM) {
-        float l = INFINITY, dl = 0.f;
-        if (q0 + tid < p.Lq) {
-          l = lse2[rows0 + q0 + tid];
-          dl = delta[rows0 + q0 + tid];
-          if (l == -INFINITY) l = INFINITY;
-        }
-        lse_s[tid] = l;
-        del_s[tid] = dl;
+        lse_s[tid] = lreg;
+        del_s[tid] = dreg;
       }
       __syncthreads();
+      if (it + 1 < nt) load_tile(t_nxt * BM);
+      t_cur = t_nxt;
+      if (it + 2 < nt) t_nxt = tile_at(it + 2);
 
       const int qbase_w = wq * 64;
       float16_t sacc[2], dpacc[2];
@@ -297,32 +338,52 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
           dpacc[mb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + 16 * s), vf[s], dpacc[mb]);
         }
       }
-      vec8 pf[4], dsf[4];
+      // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
+      float16_t gacc[2];
+      const int ql0 = qbase_w + 4 * g;  // local row of block 0, register 0
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
-        const int ql = qbase_w + mb * 32 + 4 * g;  // local row of register 0
+        const int ql = ql0 + 32 * mb;
         sm.tileT(q0 + ql, kv_col);
 #pragma unroll
         for (int rr = 0; rr < 4; rr++) {
           const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
           const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
+          for (int e = 0; e < 4; e += 2) {
             const int r = 4 * rr + e;
-            float s = sacc[mb][r];
-            if (ROUND_S) s = round_through<T>(s);
-            float x = sm.apply(s, acc_row(r));
-            if (masked) {
-              const int qi = q0 + ql + acc_row(r);
-              x = (qi < p.Lq && visible(qi, kv_col)) ? x : -INFINITY;
+            float s0 = sacc[mb][r], s1 = sacc[mb][r + 1];
+            if (ROUND_S) round_pair<T>(s0, s1);
+            sacc[mb][r] = sm.apply_sub(s0, acc_row(r), l4[e]);
+            sacc[mb][r + 1] = sm.apply_sub(s1, acc_row(r + 1), l4[e + 1]);
+            dpacc[mb][r] -= d4[e];
+            dpacc[mb][r + 1] -= d4[e + 1];
+            if (!Score2<KIND>::kGradOne) {
+              gacc[mb][r] = sm.grad(s0, acc_row(r));
+              gacc[mb][r + 1] = sm.grad(s1, acc_row(r + 1));
             }
-            float pr = fast_exp2(x - l4[e]);
-            float ds = pr * (dpacc[mb][r] - d4[e]) * (sm.grad(s, acc_row(r)) * p.scale);
-            pf[2 * mb + r / 8][r % 8] = (T)pr;
-            dsf[2 * mb + r / 8][r % 8] = (T)ds;
           }
         }
       }
+      if (masked) mask_tile_kv(sacc, p.mask, visible, q0 + ql0, kv_col, p.Lq, p.Lkv);
+      vec8 pf[4], dsf[4];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+          typename Pair<T>::v2 pp[4], dd[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int r = 8 * tt + 2 * e;
+            const float p0 = fast_exp2(sacc[mb][r]), p1 = fast_exp2(sacc[mb][r + 1]);
+            float d0 = p0 * dpacc[mb][r], d1 = p1 * dpacc[mb][r + 1];
+            if (!Score2<KIND>::kGradOne) { d0 *= gacc[mb][r]; d1 *= gacc[mb][r + 1]; }
+            pp[e] = Pair<T>::pack(p0, p1);
+            dd[e] = Pair<T>::pack(d0, d1);
+          }
+          pf[2 * mb + tt] = join_pairs<T>(pp[0], pp[1], pp[2], pp[3]);
+          dsf[2 * mb + tt] = join_pairs<T>(dd[0], dd[1], dd[2], dd[3]);
+        }
 #pragma unroll
       for (int t = 0; t < 4; t++) {
 #pragma unroll
@@ -362,7 +423,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rr + e;
-          pk.e[e] = (T)(dkacc[db][r] + red[((wk * 2 * DB + db) * 16 + r) * 64 + lane]);
+          pk.e[e] = (T)((dkacc[db][r] + red[((wk * 2 * DB + db) * 16 + r) * 64 + lane]) * p.scale);
           pv.e[e] = (T)(dvacc[db][r] + red[((wk * 2 * DB + DB + db) * 16 + r) * 64 + lane]);
         }
         *reinterpret_cast<uint2*>(dkp + 32 * db + 8 * rr) = pk.u;

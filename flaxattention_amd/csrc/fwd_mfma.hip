@@ -22,7 +22,7 @@ constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
 
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2) {
   typedef typename Frag<T>::vec8 vec8;
@@ -39,9 +39,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
   const int nqt = (p.Lq + BM - 1) / BM;
   const int total = nqt * p.Hq * p.B;
-  const int wid = xcd_remap(blockIdx.x, total);
-  const int qt = nqt - 1 - (wid % nqt);  // heavy (late) causal tiles first
-  const int bh = wid / nqt;
+  int rank, bh;
+  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
+  const int qt = nqt - 1 - rank;  // late query tiles see the most keys under causal masks
   const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
 
   const int q_row = qt * BM + w * 32 + i32;
@@ -114,77 +114,85 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
     for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
 
-  if (nt > 0) load_tile(tile_at(0) * BN);
+  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  int t_cur = nt > 0 ? tile_at(0) : 0;
+  int t_nxt = nt > 1 ? tile_at(1) : 0;
+  if (nt > 0) load_tile(t_cur * BN);
   for (int it = 0; it < nt; it++) {
-    const int kv0 = tile_at(it) * BN;
+    const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
     store_tile();
     __syncthreads();
-    if (it + 1 < nt) load_tile(tile_at(it + 1) * BN);
+    if (it + 1 < nt) load_tile(t_nxt * BN);
+    t_cur = t_nxt;
+    if (it + 2 < nt) t_nxt = tile_at(it + 2);
 
-    // ---- S^T = K . Q^T ----
-    float16_t sacc[2];
+    // Each 32-row half of the tile is one online-softmax step (keeps only 16
+    // score registers live, which is what lets four waves share a SIMD).
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
+      // ---- S^T = K . Q^T ----
+      float16_t sacc;
 #pragma unroll
-      for (int r = 0; r < 16; r++) sacc[nb][r] = 0.f;
+      for (int r = 0; r < 16; r++) sacc[r] = 0.f;
       const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
 #pragma unroll
       for (int s = 0; s < DS; s++) {
         vec8 a = *reinterpret_cast<const vec8*>(kp + 16 * s);
-        sacc[nb] = Frag<T>::mfma(a, qf[s], sacc[nb]);
+        sacc = Frag<T>::mfma(a, qf[s], sacc);
       }
-    }
 
-    // ---- score_mod, mask, online softmax ----
-    float mloc = -INFINITY;
+      // ---- score_mod relative to the running reference max, tile mask where needed ----
+      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+      sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-      const int kvb = kv0 + nb * 32 + 4 * g;
-      sm.tile(q_row, kvb);
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float s = sacc[nb][r];
-        if (ROUND_S) s = round_through<T>(s);
-        float x = sm.apply(s, acc_row(r));
-        if (masked) x = visible(q_row, kvb + acc_row(r)) ? x : -INFINITY;
-        sacc[nb][r] = x;
-        mloc = fmaxf(mloc, x);
+      for (int r = 0; r < 16; r += 2) {
+        float s0 = sacc[r], s1 = sacc[r + 1];
+        if (ROUND_S) round_pair<T>(s0, s1);
+        sacc[r] = sm.apply_sub(s0, acc_row(r), m_use);
+        sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use);
       }
-    }
-    const float m_new = fmaxf(m_run, xhalf_max(mloc));
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = fast_exp2(m_run - m_use);
-    m_run = m_new;
-    float lsum = 0.f;
-    vec8 pf[4];
+      if (masked) mask_block_q(sacc, p.mask, visible, q_row, kv0 + nb * 32, g, p.Lkv);
+
+      // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
+      const float m_rel = xhalf_max(block_max(sacc));
+      const bool need = (m_rel > kTau) || (m_run == -INFINITY && m_rel > -INFINITY);
+      if (__any(need)) {
+        const float delta = need ? m_rel : 0.f;
+        const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(-delta);
+        m_run = need ? (m_use + m_rel) : m_run;
+        l_run *= alpha;
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+        for (int r = 0; r < 16; r++) sacc[r] -= delta;
 #pragma unroll
-      for (int tt = 0; tt < 2; tt++)
+        for (int db = 0; db < DB; db++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-          float pe = fast_exp2(sacc[nb][8 * tt + e] - m_use);
-          lsum += pe;
-          pf[2 * nb + tt][e] = (T)pe;
+          for (int r = 0; r < 16; r++) oacc[db][r] *= alpha;
+      }
+      vec8 pf[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++) {
+        typename Pair<T>::v2 pr[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float p0 = fast_exp2(sacc[8 * tt + 2 * e]);
+          const float p1 = fast_exp2(sacc[8 * tt + 2 * e + 1]);
+          pr[e] = Pair<T>::pack(p0, p1);
+          l_run = Pair<T>::add_sum(pr[e], l_run);
         }
-    l_run = l_run * alpha + lsum;
-    if (__any(alpha != 1.f)) {
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) oacc[db][r] *= alpha;
-    }
+        pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+      }
 
-    // ---- O^T += V^T . P^T ----
+      // ---- O^T += V^T . P^T ----
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
+      for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
-      for (int db = 0; db < DB; db++) {
-        const T* vp = Vs + (16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-        short4_t lo = lds_read_tr(vp);
-        short4_t hi = lds_read_tr(vp + 8 * ROWE);
-        oacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), pf[t], oacc[db]);
+        for (int db = 0; db < DB; db++) {
+          const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+          short4_t lo = lds_read_tr(vp);
+          short4_t hi = lds_read_tr(vp + 8 * ROWE);
+          oacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), pf[tt], oacc[db]);
+        }
       }
     }
     __syncthreads();

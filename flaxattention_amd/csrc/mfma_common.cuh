@@ -74,15 +74,18 @@ template <typename V> __device__ __forceinline__ V join8(short4_t lo, short4_t h
 template <int KIND> struct Score2;
 
 template <> struct Score2<FLEX_SCORE_IDENTITY> {
+  static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c;
   __device__ __forceinline__ void init(const FlexScoreMod&, float scale, int h) { c = scale * kLog2e; }
   __device__ __forceinline__ void tile(int q, int kvb) {}
   __device__ __forceinline__ void tileT(int qb, int kv) {}
   __device__ __forceinline__ float apply(float s, int off) const { return s * c; }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, c, -m); }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
 template <> struct Score2<FLEX_SCORE_CHECKERBOARD> {
+  static constexpr bool kGradOne = false;  // d score_mod / d score == 1 everywhere
   float c0, c1, f0, f1;  // factor (x scale x log2e) for even / odd parity
   float ce, co, fe, fo;  // the same, resolved for even / odd `off` of this lane
   int by_kv;
@@ -101,10 +104,12 @@ template <> struct Score2<FLEX_SCORE_CHECKERBOARD> {
     if (by_kv) { co = ce; fo = fe; } else { co = par ? c0 : c1; fo = par ? f0 : f1; }
   }
   __device__ __forceinline__ float apply(float s, int off) const { return s * ((off & 1) ? co : ce); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, (off & 1) ? co : ce, -m); }
   __device__ __forceinline__ float grad(float s, int off) const { return (off & 1) ? fo : fe; }
 };
 
 template <> struct Score2<FLEX_SCORE_ALIBI> {
+  static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;
   __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
     c = scale * kLog2e;
@@ -113,10 +118,12 @@ template <> struct Score2<FLEX_SCORE_ALIBI> {
   __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(q - kvb) * slope2; step = -slope2; }
   __device__ __forceinline__ void tileT(int qb, int kv) { base = (float)(qb - kv) * slope2; step = slope2; }
   __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, step, base)); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, c, fmaf((float)off, step, base - m)); }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
 template <> struct Score2<FLEX_SCORE_REL_BIAS> {
+  static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;
   __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
     c = scale * kLog2e;
@@ -125,10 +132,12 @@ template <> struct Score2<FLEX_SCORE_REL_BIAS> {
   __device__ __forceinline__ void tile(int q, int kvb) { base = (float)(kvb - q) * slope2; step = slope2; }
   __device__ __forceinline__ void tileT(int qb, int kv) { base = (float)(kv - qb) * slope2; step = -slope2; }
   __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, fmaf((float)off, step, base)); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, c, fmaf((float)off, step, base - m)); }
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
 template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
+  static constexpr bool kGradOne = false;  // d score_mod / d score == 1 everywhere
   float a, cap2, sc;  // a = 2*log2e*scale/cap, cap2 = cap*log2e
   __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
     a = 2.f * kLog2e * scale * m.p1; cap2 = m.p0 * kLog2e; sc = scale;
@@ -140,6 +149,7 @@ template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
     return 1.f - 2.f * fast_rcp(t + 1.f);
   }
   __device__ __forceinline__ float apply(float s, int off) const { return cap2 * tanh_(s); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(cap2, tanh_(s), -m); }
   __device__ __forceinline__ float grad(float s, int off) const { float t = tanh_(s); return 1.f - t * t; }
 };
 
@@ -151,13 +161,183 @@ struct Mask2 {
   __device__ __forceinline__ bool operator()(int q, int kv) const { return kv < Lkv && ev(q, kv); }
 };
 
-// XCD-aware workgroup remap: hardware deals consecutive workgroup ids round-robin
-// to the 8 XCDs, each with its own L2.  Give every XCD a contiguous range of
-// logical ids so that workgroups sharing K/V (same batch and head) share an L2.
-__device__ __forceinline__ int xcd_remap(int wid, int total) {
+// ---------------------------------------------------------------------------
+// Tile-level mask application, hoisted out of the per-element code so that the
+// unmasked path stays one straight-line block.
+// ---------------------------------------------------------------------------
+// Lane owns query row q; accumulator block nb, register r holds key
+// kv0 + 32*nb + 4*g + acc_row(r).  Hidden entries become -inf.
+__device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m, const Mask2& visible, int q, int kv0,
+                                            int g, int Lkv) {
+  if (m.kind == FLEX_MASK_BAND) {
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      const int kvb = kv0 + 32 * nb + 4 * g;
+      const int dq = q + m.q_offset - kvb;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int off = acc_row(r), d = dq - off, kv = kvb + off;
+        const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & (kv < Lkv);
+        x[nb][r] = vis ? x[nb][r] : -INFINITY;
+      }
+    }
+  } else {
+    const uint32_t* wp = visible.ev.bits_bh + (int64_t)q * visible.ev.stride_q + (kv0 >> 5);
+    const uint32_t w0 = wp[0], w1 = wp[1];
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      const uint32_t w = (nb ? w1 : w0) >> (4 * g);
+      const int kvb = kv0 + 32 * nb + 4 * g;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int off = acc_row(r);
+        const bool vis = ((w >> off) & 1u) & (kvb + off < Lkv);
+        x[nb][r] = vis ? x[nb][r] : -INFINITY;
+      }
+    }
+  }
+}
+
+// Lane owns key kv; accumulator block mb, register r holds query
+// qb(mb) + acc_row(r) with qb(mb) = q00 + 32*mb (q00 already includes 4*g).
+__device__ __forceinline__ void mask_tile_kv(float16_t (&x)[2], const FlexMask& m, const Mask2& visible, int q00, int kv,
+                                             int Lq, int Lkv) {
+  if (m.kind == FLEX_MASK_BAND) {
+    const bool kv_ok = kv < Lkv;
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++) {
+      const int qb = q00 + 32 * mb;
+      const int dq = qb + m.q_offset - kv;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int off = acc_row(r), d = dq + off;
+        const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & kv_ok & (qb + off < Lq);
+        x[mb][r] = vis ? x[mb][r] : -INFINITY;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int qi = q00 + 32 * mb + acc_row(r);
+        const bool vis = qi < Lq && visible(qi, kv);
+        x[mb][r] = vis ? x[mb][r] : -INFINITY;
+      }
+  }
+}
+
+// Pairs of 16-bit values: packed conversion and a fused row-sum.
+template <typename T> struct Pair;
+template <> struct Pair<f16> {
+  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ v2 pack(float a, float b) { v2 h = {(_Float16)a, (_Float16)b}; return h; }
+  static __device__ __forceinline__ float add_sum(v2 h, float acc) {
+    const v2 one = {(_Float16)1.f, (_Float16)1.f};
+    return __builtin_amdgcn_fdot2(h, one, acc, false);
+  }
+};
+template <> struct Pair<bf16> {
+  typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ v2 pack(float a, float b) { v2 h = {(__bf16)a, (__bf16)b}; return h; }
+  static __device__ __forceinline__ float add_sum(v2 h, float acc) {
+    const v2 one = {(__bf16)1.f, (__bf16)1.f};
+    return __builtin_amdgcn_fdot2_f32_bf16(h, one, acc, false);
+  }
+};
+// Round two fp32 values through T with ONE packed conversion.  The empty asm
+// keeps the pair opaque so that the compiler does not split it back into two
+// scalar conversions; widening back to fp32 then fuses into the consumer
+// (v_fma_mix_f32 reads either half of an f16 pair as an operand).  No real
+// instruction is hidden inside asm here: MFMA results must only ever be read by
+// instructions the compiler's hazard handling can see.
+template <typename T> __device__ __forceinline__ typename Pair<T>::v2 round_pack(float a, float b) {
+  typedef float f2 __attribute__((ext_vector_type(2)));
+  const f2 ab = {a, b};
+  typename Pair<T>::v2 h = __builtin_convertvector(ab, typename Pair<T>::v2);
+  unsigned u = __builtin_bit_cast(unsigned, h);
+  asm("" : "+v"(u));
+  return __builtin_bit_cast(typename Pair<T>::v2, u);
+}
+template <typename T> __device__ __forceinline__ void round_pair(float& a, float& b) {
+  typename Pair<T>::v2 h = round_pack<T>(a, b);
+  a = (float)h[0];
+  b = (float)h[1];
+}
+// three-input max without the NaN-quieting canonicalisation the compiler adds to fmaxf
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+template <typename T> __device__ __forceinline__ typename Frag<T>::vec8 join_pairs(typename Pair<T>::v2 a, typename Pair<T>::v2 b,
+                                                                                    typename Pair<T>::v2 c, typename Pair<T>::v2 d) {
+  auto ab = __builtin_shufflevector(a, b, 0, 1, 2, 3);
+  auto cd = __builtin_shufflevector(c, d, 0, 1, 2, 3);
+  return __builtin_shufflevector(ab, cd, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+
+// one 32-key block: register r holds key kv0 + 4*g + acc_row(r)
+__device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
+                                             int Lkv) {
+  const int kvb = kv0 + 4 * g;
+  if (m.kind == FLEX_MASK_BAND) {
+    const int dq = q + m.q_offset - kvb;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int off = acc_row(r), d = dq - off, kv = kvb + off;
+      const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & (kv < Lkv);
+      x[r] = vis ? x[r] : -INFINITY;
+    }
+  } else {
+    const uint32_t w = visible.ev.bits_bh[(int64_t)q * visible.ev.stride_q + (kv0 >> 5)] >> (4 * g);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int off = acc_row(r);
+      const bool vis = ((w >> off) & 1u) & (kvb + off < Lkv);
+      x[r] = vis ? x[r] : -INFINITY;
+    }
+  }
+}
+__device__ __forceinline__ float block_max(const float16_t& x) {
+  float a = max3(x[0], x[1], x[2]), b = max3(x[3], x[4], x[5]);
+#pragma unroll
+  for (int r = 6; r < 14; r += 4) {
+    a = max3(a, x[r], x[r + 1]);
+    b = max3(b, x[r + 2], x[r + 3]);
+  }
+  return max3(max3(a, b, x[14]), x[15], x[15]);
+}
+
+// maximum of the 32 accumulator values of a lane: two independent chains of v_max3
+__device__ __forceinline__ float tile_max(const float16_t (&x)[2]) {
+  float a = max3(x[0][0], x[0][1], x[0][2]), b = max3(x[1][0], x[1][1], x[1][2]);
+#pragma unroll
+  for (int r = 3; r < 15; r += 2) {
+    a = max3(a, x[0][r], x[0][r + 1]);
+    b = max3(b, x[1][r], x[1][r + 1]);
+  }
+  return max3(max3(a, b, x[0][15]), x[1][15], x[1][15]);
+}
+
+// XCD-aware, heavy-first workgroup map.  Hardware deals consecutive workgroup ids
+// round-robin to the 8 XCDs (each has its own L2) and starts them in id order as
+// slots free up.  Every XCD gets a contiguous share of the (batch, head) pairs, so
+// workgroups that read the same K/V meet in one L2; inside an XCD the ids run
+// tile-major -- all heads' heaviest tile first, then the next heaviest -- so that
+// under causal-like masks the long workgroups start first and the short ones fill
+// the tail.  `rank` counts tiles from the heaviest (0) to the lightest (ntile-1).
+__device__ __forceinline__ void xcd_tile_map(int wid, int ntile, int nbh, int& rank, int& bh) {
   constexpr int kXcd = 8;
-  if (total % kXcd != 0) return wid;
-  return (wid % kXcd) * (total / kXcd) + wid / kXcd;
+  if (nbh % kXcd == 0) {
+    const int per = nbh / kXcd;           // heads per XCD
+    const int xcd = wid % kXcd, local = wid / kXcd;
+    rank = local / per;
+    bh = xcd * per + local % per;
+  } else {
+    rank = wid / nbh;
+    bh = wid % nbh;
+  }
 }
 
 }  // namespace flex
