@@ -22,7 +22,7 @@ namespace flex {
 constexpr int kStep = 32;  // KV rows per wave step
 
 template <typename T, int D, int KIND, bool ROUND_S, int NB>
-__global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : 1) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits) {
@@ -32,7 +32,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, con
   __shared__ float mbuf[4][NB][32];
   __shared__ __align__(16) float red[4][16][64];
 
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, provably uniform: step addresses stay scalar
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
   const int split = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
   const int G = p.Hq / p.Hkv;
@@ -82,25 +83,24 @@ __global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, con
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
+  // Loads of a step: scalar base (kbase + kv0 * stride) plus small per-lane
+  // offsets.  Rows past the end are clamped to the last row: their scores are
+  // masked out and their P is 0, so what they hold does not matter as long as
+  // it is finite.
+  const int last = p.Lkv - 1;
   vec8 kfr[DS];
-  uint4 vreg[NV];
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 vreg[NV];
   auto load_step = [&](int kv0) {
-    const int kr = kv0 + i32;
-    if (kr < p.Lkv) {
-      const T* kp = kbase + (int64_t)kr * ks2 + 8 * g;
+    const int lim = last - kv0;  // last valid row of this step, relative
+    const T* kp = kbase + (int64_t)kv0 * ks2 + min(i32, lim) * (int)ks2 + 8 * g;
 #pragma unroll
-      for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
-    } else {
-#pragma unroll
-      for (int s = 0; s < DS; s++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) kfr[s][e] = (T)0.f;
-    }
+    for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+    const T* vp = vbase + (int64_t)kv0 * vs2;
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + 64 * j, r = c / CPR, cc = c % CPR;
-      vreg[j] = (kv0 + r < p.Lkv) ? *reinterpret_cast<const uint4*>(vbase + (int64_t)(kv0 + r) * vs2 + cc * 8)
-                                  : make_uint4(0, 0, 0, 0);
+      vreg[j] = *reinterpret_cast<const u32x4*>(vp + min(r, lim) * (int)vs2 + cc * 8);
     }
   };
 
@@ -119,62 +119,84 @@ __global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, con
   }
   const bool trivial_mask = p.mask.kind == FLEX_MASK_BAND && p.mask.lo == INT32_MIN && p.mask.hi == INT32_MAX;
   T* Vw = Vs[w];
+  constexpr float kTau = 8.f;
 
+  // KV offsets are looked up two visits ahead so that the (dependent) tile-index
+  // load never sits between a wave and its next K/V loads
   int st = st_begin + w;
-  if (st < st_end) load_step(step_kv0(st));
+  int kv_cur = st < st_end ? step_kv0(st) : 0;
+  int kv_nx1 = st + 4 < st_end ? step_kv0(st + 4) : 0;
+  int kv_nx2 = st + 8 < st_end ? step_kv0(st + 8) : 0;
+  if (st < st_end) load_step(kv_cur);
   for (; st < st_end; st += 4) {
-    const int kv0 = step_kv0(st);
-    vec8 kcur[DS];
+    const int kv0 = kv_cur;
+    // scores first: they consume the K registers, which the next step's loads then reuse
+    float16_t s_a, s_b;  // named (not an array) so that they stay in registers
 #pragma unroll
-    for (int s = 0; s < DS; s++) kcur[s] = kfr[s];
+    for (int r = 0; r < 16; r++) { s_a[r] = 0.f; s_b[r] = 0.f; }
+#pragma unroll
+    for (int s = 0; s < DS; s++) {
+      s_a = Frag<T>::mfma(kfr[s], qf[0][s], s_a);
+      if (NB > 1) s_b = Frag<T>::mfma(kfr[s], qf[NB - 1][s], s_b);
+    }
 #pragma unroll
     for (int j = 0; j < NV; j++) {
       const int c = lane + 64 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint4*>(Vw + r * ROWE + cc * 8) = vreg[j];
+      *reinterpret_cast<u32x4*>(Vw + r * ROWE + cc * 8) = vreg[j];
     }
-    if (st + 4 < st_end) load_step(step_kv0(st + 4));
+    if (st + 4 < st_end) load_step(kv_nx1);
+    kv_cur = kv_nx1;
+    kv_nx1 = kv_nx2;
+    if (st + 12 < st_end) kv_nx2 = step_kv0(st + 12);
     const bool need_mask = !trivial_mask || (kv0 + kStep > p.Lkv);
 
     vec8 pf[NB][2];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) {
-      float16_t sacc;
+      float16_t sacc = nb ? s_b : s_a;
+      const float m_use = (m_run[nb] == -INFINITY) ? 0.f : m_run[nb];
+      sm[nb].tile(col_q[nb], kv0 + 4 * g);
 #pragma unroll
-      for (int r = 0; r < 16; r++) sacc[r] = 0.f;
-#pragma unroll
-      for (int s = 0; s < DS; s++) sacc = Frag<T>::mfma(kcur[s], qf[nb][s], sacc);
-      const int kvb = kv0 + 4 * g;
-      sm[nb].tile(col_q[nb], kvb);
-      Mask2 visible(p.mask, b, col_h[nb], p.Lkv);
-      float mloc = -INFINITY;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float s = sacc[r];
-        if (ROUND_S) s = round_through<T>(s);
-        float x = sm[nb].apply(s, acc_row(r));
-        if (need_mask) x = visible(col_q[nb], kvb + acc_row(r)) ? x : -INFINITY;
-        sacc[r] = x;
-        mloc = fmaxf(mloc, x);
+      for (int r = 0; r < 16; r += 2) {
+        float s0 = sacc[r], s1 = sacc[r + 1];
+        if (ROUND_S) round_pair<T>(s0, s1);
+        sacc[r] = sm[nb].apply_sub(s0, acc_row(r), m_use);
+        sacc[r + 1] = sm[nb].apply_sub(s1, acc_row(r + 1), m_use);
       }
-      const float m_new = fmaxf(m_run[nb], xhalf_max(mloc));
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[nb] - m_use);
-      m_run[nb] = m_new;
-      float lsum = 0.f;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float pe = fast_exp2(sacc[r] - m_use);
-        lsum += pe;
-        pf[nb][r / 8][r % 8] = (T)pe;
+      if (need_mask) {
+        Mask2 visible(p.mask, b, col_h[nb], p.Lkv);
+        mask_block_q(sacc, p.mask, visible, col_q[nb], kv0, g, p.Lkv);
       }
-      l_run[nb] = l_run[nb] * alpha + lsum;
+      // online softmax; the reference max moves only when it is beaten by 2^kTau
+      const float m_rel = xhalf_max(block_max(sacc));
+      const bool need = (m_rel > kTau) || (m_run[nb] == -INFINITY && m_rel > -INFINITY);
+      if (__any(need)) {
+        const float delta = need ? m_rel : 0.f;
+        const float alpha = (m_run[nb] == -INFINITY) ? 0.f : fast_exp2(-delta);
+        m_run[nb] = need ? (m_use + m_rel) : m_run[nb];
+        l_run[nb] *= alpha;
 #pragma unroll
-      for (int db = 0; db < DB; db++)
+        for (int r = 0; r < 16; r++) sacc[r] -= delta;
 #pragma unroll
-        for (int r = 0; r < 16; r++) oacc[nb][db][r] *= alpha;
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[nb][db][r] *= alpha;
+      }
+#pragma unroll
+      for (int tt = 0; tt < 2; tt++) {
+        typename Pair<T>::v2 pr[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float p0 = fast_exp2(sacc[8 * tt + 2 * e]);
+          const float p1 = fast_exp2(sacc[8 * tt + 2 * e + 1]);
+          pr[e] = Pair<T>::pack(p0, p1);
+          l_run[nb] = Pair<T>::add_sum(pr[e], l_run[nb]);
+        }
+        pf[nb][tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+      }
     }
-    // V strip was written by this wave only: wait for its LDS writes, no workgroup barrier
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    // the V strip was written by this wave only and LDS operations of one wave
+    // complete in order: no workgroup barrier is needed before reading it back
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int t = 0; t < 2; t++) {
@@ -186,7 +208,6 @@ __global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, con
         for (int nb = 0; nb < NB; nb++) oacc[nb][db] = Frag<T>::mfma(a, pf[nb][t], oacc[nb][db]);
       }
     }
-    __builtin_amdgcn_s_waitcnt(0xc07f);
     __builtin_amdgcn_wave_barrier();
   }
 
@@ -249,7 +270,10 @@ __global__ __launch_bounds__(256) void decode_split_kernel(FlexAttnParams p, con
   }
 }
 
-// one wave per output row: merge the splits, normalise, write O and lse2
+// one wave per output row: merge the splits, normalise, write O and lse2.
+// Lane s first takes split s's (m, l) so that the max and the weights come from
+// one round of loads; the partial outputs are then fetched with all loads in
+// flight together.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void decode_combine_kernel(FlexAttnParams p, const float* __restrict__ o_part,
                                                               const float* __restrict__ ml_part, int splits,
@@ -258,17 +282,33 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(FlexAttnParams p, c
   const int64_t rows = (int64_t)p.B * p.Hq * p.Lq;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
-  float m = -INFINITY;
-  for (int s = 0; s < splits; s++) m = fmaxf(m, ml_part[(s * rows + row) * 2]);
-  float l = 0.f, acc[D / 64];
+  float ms = -INFINITY, ls = 0.f;
+  if (lane < splits) {
+    const float2 ml = *reinterpret_cast<const float2*>(ml_part + (lane * rows + row) * 2);
+    ms = ml.x;
+    ls = ml.y;
+  }
+  float m = ms;
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  const float sc = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m);
+  float l = sc * ls;
+  for (int off = 32; off > 0; off >>= 1) l += __shfl_xor(l, off, 64);
+  float acc[D / 64];
 #pragma unroll
   for (int a = 0; a < D / 64; a++) acc[a] = 0.f;
-  for (int s = 0; s < splits; s++) {
-    const float ms = ml_part[(s * rows + row) * 2];
-    const float sc = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m);
-    l += sc * ml_part[(s * rows + row) * 2 + 1];
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float v[8][D / 64];
 #pragma unroll
-    for (int a = 0; a < D / 64; a++) acc[a] += sc * o_part[(s * rows + row) * D + lane + 64 * a];
+    for (int u = 0; u < 8; u++)
+#pragma unroll
+      for (int a = 0; a < D / 64; a++)
+        v[u][a] = (s0 + u < splits) ? o_part[((s0 + u) * rows + row) * D + lane + 64 * a] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const float w = __shfl(sc, s0 + u, 64);
+#pragma unroll
+      for (int a = 0; a < D / 64; a++) acc[a] = fmaf(w, v[u][a], acc[a]);
+    }
   }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   const int qi = (int)(row % p.Lq);
@@ -325,10 +365,10 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 }
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
-  // aim for about four workgroups per CU (256 CUs), at least 8 steps per workgroup
+  // aim for three workgroups per CU (256 CUs; the kernel fits three waves per SIMD), at least 8 steps each
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
-  int s = (int)((1024 + heads - 1) / heads);
+  int s = (int)((768 + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
   if (s > 64) s = 64;
@@ -346,7 +386,7 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
     flex_set_error("decode needs 16-byte aligned tensors");
     return 1;
   }
-  if (splits > 65535) { flex_set_error("decode: too many splits (%d)", splits); return 1; }
+  if (splits > 64) { flex_set_error("decode: at most 64 splits (got %d)", splits); return 1; }
   const size_t rows = (size_t)p.B * p.Hq * p.Lq;
   float* o_part = (float*)workspace;
   float* ml_part = o_part + rows * splits * p.D;

@@ -164,38 +164,53 @@ struct Mask2 {
 // ---------------------------------------------------------------------------
 // Tile-level mask application, hoisted out of the per-element code so that the
 // unmasked path stays one straight-line block.
+//
+// Band masks: with d = q + q_offset - kv, a key is visible iff
+//     d >= lo  &&  (d <= hi || kv <= sink)  &&  kv < Lkv.
+// Inside a 32-key block a register's key is kvb + off with `off` a compile-time
+// constant, so every condition becomes a comparison of `off` with a per-lane
+// bound:  off <= up  &&  (off >= wlo || off <= snk).  Bounds are clamped to
+// +-2^30 so that no subtraction overflows (sequence positions are far smaller).
 // ---------------------------------------------------------------------------
-// Lane owns query row q; accumulator block nb, register r holds key
-// kv0 + 32*nb + 4*g + acc_row(r).  Hidden entries become -inf.
-__device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m, const Mask2& visible, int q, int kv0,
-                                            int g, int Lkv) {
+constexpr int kBig = 1 << 30;
+__device__ __forceinline__ int clamp_big(int x) { return min(max(x, -kBig), kBig); }
+
+// one 32-key block: register r holds key kv0 + 4*g + acc_row(r); lane owns query q
+__device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
+                                             int Lkv) {
+  const int kvb = kv0 + 4 * g;
   if (m.kind == FLEX_MASK_BAND) {
+    const int dq = q + m.q_offset - kvb;                           // d at off = 0; d = dq - off
+    const int up = min(dq - clamp_big(m.lo), Lkv - 1 - kvb);       // off <= up  <=>  d >= lo && kv < Lkv
+    if (m.hi >= kBig) {
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-      const int kvb = kv0 + 32 * nb + 4 * g;
-      const int dq = q + m.q_offset - kvb;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int off = acc_row(r), d = dq - off, kv = kvb + off;
-        const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & (kv < Lkv);
-        x[nb][r] = vis ? x[nb][r] : -INFINITY;
-      }
-    }
-  } else {
-    const uint32_t* wp = visible.ev.bits_bh + (int64_t)q * visible.ev.stride_q + (kv0 >> 5);
-    const uint32_t w0 = wp[0], w1 = wp[1];
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
-      const uint32_t w = (nb ? w1 : w0) >> (4 * g);
-      const int kvb = kv0 + 32 * nb + 4 * g;
+      for (int r = 0; r < 16; r++) x[r] = (acc_row(r) <= up) ? x[r] : -INFINITY;
+    } else {
+      const int wlo = dq - m.hi;                                    // off >= wlo <=> d <= hi
+      const int snk = clamp_big(m.sink) - kvb;                      // off <= snk <=> kv <= sink
 #pragma unroll
       for (int r = 0; r < 16; r++) {
         const int off = acc_row(r);
-        const bool vis = ((w >> off) & 1u) & (kvb + off < Lkv);
-        x[nb][r] = vis ? x[nb][r] : -INFINITY;
+        const bool vis = (off <= up) & ((off >= wlo) | (off <= snk));
+        x[r] = vis ? x[r] : -INFINITY;
       }
     }
+  } else {
+    const uint32_t w = visible.ev.bits_bh[(int64_t)q * visible.ev.stride_q + (kv0 >> 5)] >> (4 * g);
+    const int up = Lkv - 1 - kvb;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int off = acc_row(r);
+      const bool vis = ((w >> off) & 1u) & (off <= up);
+      x[r] = vis ? x[r] : -INFINITY;
+    }
   }
+}
+// a 64-key tile = two blocks
+__device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m, const Mask2& visible, int q, int kv0,
+                                            int g, int Lkv) {
+  mask_block_q(x[0], m, visible, q, kv0, g, Lkv);
+  mask_block_q(x[1], m, visible, q, kv0 + 32, g, Lkv);
 }
 
 // Lane owns key kv; accumulator block mb, register r holds query
@@ -204,14 +219,19 @@ __device__ __forceinline__ void mask_tile_kv(float16_t (&x)[2], const FlexMask& 
                                              int Lq, int Lkv) {
   if (m.kind == FLEX_MASK_BAND) {
     const bool kv_ok = kv < Lkv;
+    const bool sunk = kv <= m.sink;
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
       const int qb = q00 + 32 * mb;
-      const int dq = qb + m.q_offset - kv;
+      const int dq = qb + m.q_offset - kv;                          // d = dq + off
+      const int lo_off = clamp_big(m.lo) - dq;                      // off >= lo_off <=> d >= lo
+      const int up = kv_ok ? (Lq - 1 - qb) : -1;                    // off <= up <=> q < Lq (and the key exists)
+      const int whi = sunk ? kBig : (clamp_big(m.hi) - dq);         // off <= whi <=> d <= hi || kv <= sink
+      const int hi_off = min(up, whi);
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const int off = acc_row(r), d = dq + off;
-        const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & kv_ok & (qb + off < Lq);
+        const int off = acc_row(r);
+        const bool vis = (off >= lo_off) & (off <= hi_off);
         x[mb][r] = vis ? x[mb][r] : -INFINITY;
       }
     }
@@ -277,28 +297,6 @@ template <typename T> __device__ __forceinline__ typename Frag<T>::vec8 join_pai
   return __builtin_shufflevector(ab, cd, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
-// one 32-key block: register r holds key kv0 + 4*g + acc_row(r)
-__device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
-                                             int Lkv) {
-  const int kvb = kv0 + 4 * g;
-  if (m.kind == FLEX_MASK_BAND) {
-    const int dq = q + m.q_offset - kvb;
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int off = acc_row(r), d = dq - off, kv = kvb + off;
-      const bool vis = (d >= m.lo) & ((d <= m.hi) | (kv <= m.sink)) & (kv < Lkv);
-      x[r] = vis ? x[r] : -INFINITY;
-    }
-  } else {
-    const uint32_t w = visible.ev.bits_bh[(int64_t)q * visible.ev.stride_q + (kv0 >> 5)] >> (4 * g);
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int off = acc_row(r);
-      const bool vis = ((w >> off) & 1u) & (kvb + off < Lkv);
-      x[r] = vis ? x[r] : -INFINITY;
-    }
-  }
-}
 __device__ __forceinline__ float block_max(const float16_t& x) {
   float a = max3(x[0], x[1], x[2]), b = max3(x[3], x[4], x[5]);
 #pragma unroll
