@@ -13,8 +13,9 @@
 //  bwd_dkv_kernel  one workgroup per 64 key rows, sweeping query tiles of 128
 //                  from the transposed tile lists.  Here a lane owns one key
 //                  row: S = Q.K^T, dP = dO.V^T, dV^T += dO^T.P, dK^T += Q^T.dS.
-//                  Waves 0/1 and 2/3 split the query tile and are summed through
-//                  LDS at the end.  With GQA the workgroup loops over the query
+//                  Eight waves = 2 key blocks x 4 query quarters (two waves per
+//                  SIMD, so one wave's MFMA overlaps the other's vector work);
+//                  the quarters are summed through LDS at the end.  With GQA the workgroup loops over the query
 //                  heads of its group.
 #include "mfma_common.cuh"
 
@@ -211,16 +212,29 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
 
 extern __shared__ __align__(16) unsigned char bwd_smem[];
 
+// dK/dV workgroup: 2 key blocks x NQG query groups.  D = 64 runs 8 waves (two per
+// SIMD, so one wave's MFMA overlaps the other's vector work); D = 128 needs the
+// registers of a full SIMD per wave and runs 4 waves, each taking two 32-row
+// query blocks in turn.
+template <int D> struct DkvShape {
+  static constexpr int kWaves = D == 64 ? 8 : 4;
+  static constexpr int kThreads = kWaves * 64;
+  static constexpr int kNQG = kWaves / 2;        // query groups
+  static constexpr int kQBlocks = 4 / kNQG;      // 32-row query blocks per wave and tile
+};
+
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
-                                                       const T* __restrict__ k, const T* __restrict__ v,
-                                                       const float* __restrict__ lse2,
-                                                       const float* __restrict__ delta,
-                                                       const T* __restrict__ d_o, T* __restrict__ dk,
-                                                       T* __restrict__ dv) {
+__global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                               const T* __restrict__ k, const T* __restrict__ v,
+                                                               const float* __restrict__ lse2,
+                                                               const float* __restrict__ delta,
+                                                               const T* __restrict__ d_o, T* __restrict__ dk,
+                                                               T* __restrict__ dv) {
   typedef typename Frag<T>::vec8 vec8;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int BM = kBM, BN = kBN;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / 256;
+  constexpr int kDkvThreads = DkvShape<D>::kThreads, NQG = DkvShape<D>::kNQG, QBW = DkvShape<D>::kQBlocks;
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
   T* Qs = reinterpret_cast<T*>(bwd_smem);
   T* Os = Qs + BM * ROWE;
   float* lse_s = reinterpret_cast<float*>(Os + BM * ROWE);
@@ -228,9 +242,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
-  const int wk = w & 1, wq = w >> 1;
+  const int wk = w & 1, wq = w >> 1;  // key block (32 rows) and query group of this wave
   const int nkt = (p.Lkv + BN - 1) / BN;
-  const int total = nkt * p.Hkv * p.B;
   int kt, bh;  // early key tiles see the most queries under causal masks
   xcd_tile_map(blockIdx.x, nkt, p.Hkv * p.B, kt, bh);
   const int hk = bh % p.Hkv, b = bh / p.Hkv, G = p.Hq / p.Hkv;
@@ -281,18 +294,14 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
       if (!full_idx) return it;
       return it < n_full ? full_idx[it] : part_idx[it - n_full];
     };
-    uint4 qreg[NLD], oreg[NLD];
+    u32x4 qreg[NLD], oreg[NLD];
     float lreg = INFINITY, dreg = 0.f;
     auto load_tile = [&](int q0) {
 #pragma unroll
       for (int j = 0; j < NLD; j++) {
-        int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-        qreg[j] = make_uint4(0, 0, 0, 0);
-        oreg[j] = make_uint4(0, 0, 0, 0);
-        if (q0 + r < p.Lq) {
-          qreg[j] = *reinterpret_cast<const uint4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
-          oreg[j] = *reinterpret_cast<const uint4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
-        }
+        const int c = tid + kDkvThreads * j, r = min(c / CPR, p.Lq - 1 - q0), cc = c % CPR;  // clamped: finite filler
+        qreg[j] = *reinterpret_cast<const u32x4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
+        oreg[j] = *reinterpret_cast<const u32x4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
       }
       lreg = INFINITY;
       dreg = 0.f;
@@ -311,12 +320,12 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
       __syncthreads();  // previous tile fully consumed
 #pragma unroll
       for (int j = 0; j < NLD; j++) {
-        int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-        *reinterpret_cast<uint4*>(Qs + r * ROWE + cc * 8) = qreg[j];
-        *reinterpret_cast<uint4*>(Os + r * ROWE + cc * 8) = oreg[j];
+        const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
+        *reinterpret_cast<u32x4*>(Qs + r * ROWE + cc * 8) = qreg[j];
+        *reinterpret_cast<u32x4*>(Os + r * ROWE + cc * 8) = oreg[j];
       }
       if (tid < BM) {
-        lse_s[tid] = lreg;
+        lse_s[tid] = lreg;   // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
         del_s[tid] = dreg;
       }
       __syncthreads();
@@ -324,93 +333,108 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
       t_cur = t_nxt;
       if (it + 2 < nt) t_nxt = tile_at(it + 2);
 
-      const int qbase_w = wq * 64;
-      float16_t sacc[2], dpacc[2];
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++) {
+      for (int qs = 0; qs < QBW; qs++) {
+      // ---- S = Q.K^T and dP = dO.V^T for 32 query rows x 32 keys ----
+      const int qrow_w = (wq * QBW + qs) * 32;
+      float16_t sacc, dpacc;
 #pragma unroll
-        for (int r = 0; r < 16; r++) { sacc[mb][r] = 0.f; dpacc[mb][r] = 0.f; }
-        const T* qp = Qs + (qbase_w + mb * 32 + i32) * ROWE + 8 * g;
-        const T* op = Os + (qbase_w + mb * 32 + i32) * ROWE + 8 * g;
+      for (int r = 0; r < 16; r++) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+      {
+        const T* qp = Qs + (qrow_w + i32) * ROWE + 8 * g;
+        const T* op = Os + (qrow_w + i32) * ROWE + 8 * g;
 #pragma unroll
         for (int s = 0; s < DS; s++) {
-          sacc[mb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + 16 * s), kf[s], sacc[mb]);
-          dpacc[mb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + 16 * s), vf[s], dpacc[mb]);
+          sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + 16 * s), kf[s], sacc);
+          dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + 16 * s), vf[s], dpacc);
         }
       }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
-      float16_t gacc[2];
-      const int ql0 = qbase_w + 4 * g;  // local row of block 0, register 0
+      float16_t gacc;
+      const int ql = qrow_w + 4 * g;  // local row of register 0
+      sm.tileT(q0 + ql, kv_col);
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++) {
-        const int ql = ql0 + 32 * mb;
-        sm.tileT(q0 + ql, kv_col);
+      for (int rr = 0; rr < 4; rr++) {
+        const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
+        const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
 #pragma unroll
-        for (int rr = 0; rr < 4; rr++) {
-          const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
-          const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
-#pragma unroll
-          for (int e = 0; e < 4; e += 2) {
-            const int r = 4 * rr + e;
-            float s0 = sacc[mb][r], s1 = sacc[mb][r + 1];
-            if (ROUND_S) round_pair<T>(s0, s1);
-            sacc[mb][r] = sm.apply_sub(s0, acc_row(r), l4[e]);
-            sacc[mb][r + 1] = sm.apply_sub(s1, acc_row(r + 1), l4[e + 1]);
-            dpacc[mb][r] -= d4[e];
-            dpacc[mb][r + 1] -= d4[e + 1];
-            if (!Score2<KIND>::kGradOne) {
-              gacc[mb][r] = sm.grad(s0, acc_row(r));
-              gacc[mb][r + 1] = sm.grad(s1, acc_row(r + 1));
-            }
+        for (int e = 0; e < 4; e += 2) {
+          const int r = 4 * rr + e;
+          float s0 = sacc[r], s1 = sacc[r + 1];
+          if (ROUND_S) round_pair<T>(s0, s1);
+          sacc[r] = sm.apply_sub(s0, acc_row(r), l4[e]);
+          sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), l4[e + 1]);
+          dpacc[r] -= d4[e];
+          dpacc[r + 1] -= d4[e + 1];
+          if (!Score2<KIND>::kGradOne) {
+            gacc[r] = sm.grad(s0, acc_row(r));
+            gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
           }
         }
       }
-      if (masked) mask_tile_kv(sacc, p.mask, visible, q0 + ql0, kv_col, p.Lq, p.Lkv);
-      vec8 pf[4], dsf[4];
+      if (masked) mask_block_kv(sacc, p.mask, visible, q0 + ql, kv_col, p.Lq, p.Lkv);
+      vec8 pf[2], dsf[2];
 #pragma unroll
-      for (int mb = 0; mb < 2; mb++)
+      for (int tt = 0; tt < 2; tt++) {
+        typename Pair<T>::v2 pp[4], dd[4];
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-          typename Pair<T>::v2 pp[4], dd[4];
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const int r = 8 * tt + 2 * e;
-            const float p0 = fast_exp2(sacc[mb][r]), p1 = fast_exp2(sacc[mb][r + 1]);
-            float d0 = p0 * dpacc[mb][r], d1 = p1 * dpacc[mb][r + 1];
-            if (!Score2<KIND>::kGradOne) { d0 *= gacc[mb][r]; d1 *= gacc[mb][r + 1]; }
-            pp[e] = Pair<T>::pack(p0, p1);
-            dd[e] = Pair<T>::pack(d0, d1);
-          }
-          pf[2 * mb + tt] = join_pairs<T>(pp[0], pp[1], pp[2], pp[3]);
-          dsf[2 * mb + tt] = join_pairs<T>(dd[0], dd[1], dd[2], dd[3]);
+        for (int e = 0; e < 4; e++) {
+          const int r = 8 * tt + 2 * e;
+          const float p0 = fast_exp2(sacc[r]), p1 = fast_exp2(sacc[r + 1]);
+          float d0 = p0 * dpacc[r], d1 = p1 * dpacc[r + 1];
+          if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
+          pp[e] = Pair<T>::pack(p0, p1);
+          dd[e] = Pair<T>::pack(d0, d1);
         }
+        pf[tt] = join_pairs<T>(pp[0], pp[1], pp[2], pp[3]);
+        dsf[tt] = join_pairs<T>(dd[0], dd[1], dd[2], dd[3]);
+      }
+      // ---- dV^T += dO^T.P, dK^T += Q^T.dS (contraction over this wave's 32 query rows) ----
 #pragma unroll
-      for (int t = 0; t < 4; t++) {
+      for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const int off = (qbase_w + 16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+          const int off = (qrow_w + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
           vec8 a_do = join8<vec8>(lds_read_tr(Os + off), lds_read_tr(Os + off + 8 * ROWE));
-          dvacc[db] = Frag<T>::mfma(a_do, pf[t], dvacc[db]);
+          dvacc[db] = Frag<T>::mfma(a_do, pf[tt], dvacc[db]);
           vec8 a_q = join8<vec8>(lds_read_tr(Qs + off), lds_read_tr(Qs + off + 8 * ROWE));
-          dkacc[db] = Frag<T>::mfma(a_q, dsf[t], dkacc[db]);
+          dkacc[db] = Frag<T>::mfma(a_q, dsf[tt], dkacc[db]);
         }
       }
+      }  // query blocks of this wave
     }
   }
 
-  // sum the two query halves (waves wq = 0 and 1 of the same key block) through LDS
-  __syncthreads();
-  float* red = reinterpret_cast<float*>(bwd_smem);  // [2 key blocks][2*DB*16 regs][64 lanes]
-  if (wq == 1) {
+  // sum the query groups of each key block through LDS: (3,2 -> 1,0 then) 1 -> 0
+  float* red = reinterpret_cast<float*>(bwd_smem);  // [2 slots][2 key blocks][2*DB*16 regs][64 lanes]
+  constexpr int kRegs = 2 * DB * 16;
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+  for (int round = (NQG == 4 ? 0 : 1); round < 2; round++) {
+    __syncthreads();
+    const bool writer = round == 0 ? (wq >= 2) : (wq == 1);
+    const bool reader = round == 0 ? (wq < 2) : (wq == 0);
+    const int slot = round == 0 ? (wq & 1) : 0;
+    float* base = red + ((size_t)(slot * 2 + wk) * kRegs) * 64 + lane;
+    if (writer) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        red[((wk * 2 * DB + db) * 16 + r) * 64 + lane] = dkacc[db][r];
-        red[((wk * 2 * DB + DB + db) * 16 + r) * 64 + lane] = dvacc[db][r];
-      }
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          base[(db * 16 + r) * 64] = dkacc[db][r];
+          base[((DB + db) * 16 + r) * 64] = dvacc[db][r];
+        }
+    }
+    __syncthreads();
+    if (reader) {
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          dkacc[db][r] += base[(db * 16 + r) * 64];
+          dvacc[db][r] += base[((DB + db) * 16 + r) * 64];
+        }
+    }
   }
-  __syncthreads();
   if (wq == 0 && kv_col < p.Lkv) {
     const int64_t row_id = ((int64_t)b * p.Hkv + hk) * p.Lkv + kv_col;
     T* dkp = dk + row_id * D + 4 * g;
@@ -423,8 +447,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rr + e;
-          pk.e[e] = (T)((dkacc[db][r] + red[((wk * 2 * DB + db) * 16 + r) * 64 + lane]) * p.scale);
-          pv.e[e] = (T)(dvacc[db][r] + red[((wk * 2 * DB + DB + db) * 16 + r) * 64 + lane]);
+          pk.e[e] = (T)(dkacc[db][r] * p.scale);  // the scale factor of dS is applied once here
+          pv.e[e] = (T)dvacc[db][r];
         }
         *reinterpret_cast<uint2*>(dkp + 32 * db + 8 * rr) = pk.u;
         *reinterpret_cast<uint2*>(dvp + 32 * db + 8 * rr) = pv.u;
@@ -434,7 +458,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(FlexAttnParams p, const T*
 
 template <int D, typename T> constexpr size_t dkv_smem() {
   size_t tiles = (size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float);
-  size_t red = (size_t)2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
+  size_t red = (size_t)2 * 2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
   return tiles > red ? tiles : red;
 }
 
@@ -454,7 +478,7 @@ static int launch_one(const FlexAttnParams& p, const void* q, const void* k, con
     if (e != hipSuccess) return 2;
     attr_set = true;
   }
-  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS>), dim3(nkt * p.Hkv * p.B), dim3(256), sm, s, p, (const T*)q, (const T*)k,
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p, (const T*)q, (const T*)k,
                      (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
   return 0;
 }

@@ -22,7 +22,7 @@ namespace flex {
 constexpr int kStep = 32;  // KV rows per wave step
 
 template <typename T, int D, int KIND, bool ROUND_S, int NB>
-__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : 1) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits) {

@@ -213,37 +213,28 @@ __device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m
   mask_block_q(x[1], m, visible, q, kv0 + 32, g, Lkv);
 }
 
-// Lane owns key kv; accumulator block mb, register r holds query
-// qb(mb) + acc_row(r) with qb(mb) = q00 + 32*mb (q00 already includes 4*g).
-__device__ __forceinline__ void mask_tile_kv(float16_t (&x)[2], const FlexMask& m, const Mask2& visible, int q00, int kv,
-                                             int Lq, int Lkv) {
+// Lane owns key kv; register r holds query qb + acc_row(r) (qb already includes 4*g).
+__device__ __forceinline__ void mask_block_kv(float16_t& x, const FlexMask& m, const Mask2& visible, int qb, int kv,
+                                              int Lq, int Lkv) {
   if (m.kind == FLEX_MASK_BAND) {
-    const bool kv_ok = kv < Lkv;
-    const bool sunk = kv <= m.sink;
+    const int dq = qb + m.q_offset - kv;                          // d = dq + off
+    const int lo_off = clamp_big(m.lo) - dq;                      // off >= lo_off <=> d >= lo
+    const int up = (kv < Lkv) ? (Lq - 1 - qb) : -1;               // off <= up <=> q < Lq (and the key exists)
+    const int whi = (kv <= m.sink) ? kBig : (clamp_big(m.hi) - dq);  // off <= whi <=> d <= hi || kv <= sink
+    const int hi_off = min(up, whi);
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++) {
-      const int qb = q00 + 32 * mb;
-      const int dq = qb + m.q_offset - kv;                          // d = dq + off
-      const int lo_off = clamp_big(m.lo) - dq;                      // off >= lo_off <=> d >= lo
-      const int up = kv_ok ? (Lq - 1 - qb) : -1;                    // off <= up <=> q < Lq (and the key exists)
-      const int whi = sunk ? kBig : (clamp_big(m.hi) - dq);         // off <= whi <=> d <= hi || kv <= sink
-      const int hi_off = min(up, whi);
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int off = acc_row(r);
-        const bool vis = (off >= lo_off) & (off <= hi_off);
-        x[mb][r] = vis ? x[mb][r] : -INFINITY;
-      }
+    for (int r = 0; r < 16; r++) {
+      const int off = acc_row(r);
+      const bool vis = (off >= lo_off) & (off <= hi_off);
+      x[r] = vis ? x[r] : -INFINITY;
     }
   } else {
 #pragma unroll
-    for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int qi = q00 + 32 * mb + acc_row(r);
-        const bool vis = qi < Lq && visible(qi, kv);
-        x[mb][r] = vis ? x[mb][r] : -INFINITY;
-      }
+    for (int r = 0; r < 16; r++) {
+      const int qi = qb + acc_row(r);
+      const bool vis = qi < Lq && visible(qi, kv);
+      x[r] = vis ? x[r] : -INFINITY;
+    }
   }
 }
 
