@@ -11,7 +11,7 @@ import subprocess
 from typing import Optional
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libflexattn.so")
+LIB_PATH = os.environ.get("FLEXATTN_LIB") or os.path.join(_HERE, "libflexattn.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FLEX_F32, FLEX_F16, FLEX_BF16 = 0, 1, 2
@@ -49,7 +49,8 @@ class FlexAttnParams(C.Structure):
                 ("q_stride", C.c_int64 * 3), ("k_stride", C.c_int64 * 3),
                 ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
                 ("scale", C.c_float), ("flags", C.c_int32),
-                ("score", FlexScoreMod), ("mask", FlexMask), ("tiles", FlexTileLists)]
+                ("score", FlexScoreMod), ("mask", FlexMask), ("tiles", FlexTileLists),
+                ("tiles_bwd", FlexTileLists)]
 
 
 EXPORTS = [
@@ -88,7 +89,7 @@ def lib() -> C.CDLL:
     L = C.CDLL(LIB_PATH)
     L.flexattn_abi_version.restype = C.c_int
     L.flexattn_last_error.restype = C.c_char_p
-    L.flexattn_preferred_tiles.argtypes = [C.c_int32] * 5 + [C.POINTER(C.c_int32)] * 2
+    L.flexattn_preferred_tiles.argtypes = [C.c_int32] * 6 + [C.POINTER(C.c_int32)] * 2
     L.flexattn_block_mask_workspace_bytes.restype = C.c_size_t
     L.flexattn_block_mask_workspace_bytes.argtypes = [C.c_int32] * 4
     L.flexattn_block_mask_build.argtypes = ([C.POINTER(FlexMask)] + [C.c_int32] * 6 +

@@ -86,7 +86,8 @@ class _Plan:
         self.dtype = q.dtype
         self.score, self.mask, self.block_mask = score, mask, block_mask
         self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
-        self.lists = None
+        self.lists = None       # tile lists for the forward / decode kernels
+        self.lists_bwd = None   # tile lists for the backward kernels
         self.keep = [mask.bits]
 
     def params(self, q, k, v, o) -> _lib.FlexAttnParams:
@@ -100,9 +101,9 @@ class _Plan:
         p.scale, p.flags = self.scale, self.flags
         p.score = self.score.c_struct()
         p.mask = self.mask.c_struct()
-        L = self.lists
-        if L is not None:
-            t = p.tiles
+        for L, t in ((self.lists, p.tiles), (self.lists_bwd, p.tiles_bwd)):
+            if L is None:
+                continue
             t.kv_num, t.kv_idx = L["kv_num_blocks"].data_ptr(), L["kv_indices"].data_ptr()
             t.full_kv_num, t.full_kv_idx = L["full_kv_num_blocks"].data_ptr(), L["full_kv_indices"].data_ptr()
             t.q_num, t.q_idx = L["q_num_blocks"].data_ptr(), L["q_indices"].data_ptr()
@@ -138,12 +139,18 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
                  opts.get("decode_splits", 0) if opts.get("decode", True) else 0)
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
-        qb, kvb = _lib.C.c_int32(0), _lib.C.c_int32(0)
-        _lib.lib().flexattn_preferred_tiles(_DTYPES[q.dtype], D, v.shape[3], Lq, Lkv, _lib.C.byref(qb), _lib.C.byref(kvb))
-        if qb.value > 0:
-            holder = block_mask if block_mask is not None else _holder_for(mask)
-            holder.spec = mask
-            plan.lists = holder.tile_lists(qb.value, kvb.value, B, Hq, Lq, Lkv, dev)
+        holder = block_mask if block_mask is not None else _holder_for(mask)
+        holder.spec = mask
+        for which in (0, 1):
+            qb, kvb = _lib.C.c_int32(0), _lib.C.c_int32(0)
+            _lib.lib().flexattn_preferred_tiles(_DTYPES[q.dtype], D, v.shape[3], Lq, Lkv, which,
+                                                _lib.C.byref(qb), _lib.C.byref(kvb))
+            if qb.value > 0:
+                lists = holder.tile_lists(qb.value, kvb.value, B, Hq, Lq, Lkv, dev)
+                if which == 0:
+                    plan.lists = lists
+                else:
+                    plan.lists_bwd = lists
     return plan
 
 

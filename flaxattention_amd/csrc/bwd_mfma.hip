@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* 
   float lse = lse2[row_id];
   if (lse == -INFINITY) lse = INFINITY;  // row without visible keys: P = 0
 
-  const FlexTileLists& tl = p.tiles;
+  const FlexTileLists& tl = p.tiles_bwd;
   const int32_t* full_idx = nullptr;
   const int32_t* part_idx = nullptr;
   int n_full, n_part = 0;
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
 #pragma unroll
     for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
 
-  const FlexTileLists& tl = p.tiles;
+  const FlexTileLists& tl = p.tiles_bwd;
   Score2<KIND> sm;
 
   for (int gi = 0; gi < G; gi++) {
@@ -512,7 +512,8 @@ bool flex_mfma_shape_ok(const FlexAttnParams& p);
 bool flex_mfma_bwd_supported(const FlexAttnParams& p) {
   if (!flex_mfma_shape_ok(p)) return false;
   // the dK/dV kernel needs the transposed lists whenever lists are given
-  const FlexTileLists& t = p.tiles;
+  const FlexTileLists& t = p.tiles_bwd;
+  if (t.kv_num && (t.q_block != kBM || t.kv_block != kBN)) return false;
   if (t.kv_num && (!t.q_num || !t.q_idx || !t.full_q_num || !t.full_q_idx)) return false;
   return true;
 }

@@ -28,7 +28,7 @@ int flex_decode_default_splits(const FlexAttnParams& p);
 size_t flex_decode_workspace(const FlexAttnParams& p, int splits);
 int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
                        void* workspace, hipStream_t s);
-void flex_mfma_tiles(int dtype, int D, int Dv, int* qb, int* kvb);
+void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb);
 
 static int validate(const FlexAttnParams* p, const char* who) {
   if (!p) { flex_set_error("%s: null params", who); return 1; }
@@ -44,8 +44,10 @@ static int validate(const FlexAttnParams* p, const char* who) {
   if (p->score.kind == FLEX_SCORE_TANH_SOFTCAP && !(p->score.p0 > 0.f)) { flex_set_error("%s: tanh soft-cap needs cap > 0", who); return 1; }
   if (p->mask.kind != FLEX_MASK_BAND && p->mask.kind != FLEX_MASK_BITS) { flex_set_error("%s: unknown mask kind %d", who, p->mask.kind); return 1; }
   if (p->mask.kind == FLEX_MASK_BITS && !p->mask.bits) { flex_set_error("%s: bitmap mask without bits", who); return 1; }
-  const FlexTileLists& t = p->tiles;
-  if (t.kv_num) {
+  const FlexTileLists* both[2] = {&p->tiles, &p->tiles_bwd};
+  for (int i = 0; i < 2; i++) {
+    const FlexTileLists& t = *both[i];
+    if (!t.kv_num) continue;
     if (!t.kv_idx || !t.full_kv_num || !t.full_kv_idx) { flex_set_error("%s: tile lists need kv_idx, full_kv_num and full_kv_idx", who); return 1; }
     if (t.q_block <= 0 || t.kv_block <= 0 || (int64_t)t.n_q_blocks * t.q_block < p->Lq || (int64_t)t.n_kv_blocks * t.kv_block < p->Lkv) {
       flex_set_error("%s: tile lists (%d x %d blocks of %d x %d) do not cover Lq=%d, Lkv=%d", who, t.n_q_blocks, t.n_kv_blocks, t.q_block, t.kv_block, p->Lq, p->Lkv);
@@ -64,9 +66,9 @@ static int check_launch(const char* who) {
 extern "C" int flexattn_abi_version(void) { return 1; }
 extern "C" const char* flexattn_last_error(void) { return g_err; }
 
-extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t* qb, int32_t* kvb) {
+extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t which, int32_t* qb, int32_t* kvb) {
   int a = 0, b = 0;
-  flex_mfma_tiles(dtype, D, Dv, &a, &b);
+  flex_mfma_tiles(dtype, D, Dv, which, &a, &b);
   if (qb) *qb = a;
   if (kvb) *kvb = b;
   return 0;

@@ -5,54 +5,65 @@
 // for 16-bit inputs, with a real online softmax and with skipping of masked-out
 // KV tiles, which the reference computes but never uses.
 //
-// Work decomposition: one workgroup (4 waves) per 128 query rows of one
-// (batch, head); each wave owns 32 query rows.  KV tiles of 64 rows are staged
-// through LDS (register-prefetched one tile ahead).  Per tile and wave:
-//   S^T[kv, q]  = K_tile . Q^T          8 x v_mfma_f32_32x32x16 (D = 64)
-//   online softmax in the accumulator layout: a lane holds 32 of the 64 scores
-//   of ONE query row, the other 32 sit in lane ^ 32 -> row max/sum are
-//   in-register reductions plus one permlane32 swap
-//   O^T[d, q] += V_tile^T . P^T         8 x v_mfma (P^T is already in B-operand
+// Work decomposition: one workgroup (4 waves) per BM query rows of one (batch,
+// head); each wave owns RQ blocks of 32 query rows (RQ = 2, BM = 256 for D = 64;
+// RQ = 1, BM = 128 for D = 128).  KV tiles of 64 rows go through two LDS stages
+// (register-prefetched one tile ahead, one workgroup barrier per tile).  Every K
+// and V fragment read from LDS feeds RQ MFMAs, and every K/V tile fetched from L2
+// serves BM query rows: with 128 B rows (D = 64) the kernel is otherwise bound by
+// L2->LDS and LDS->register traffic long before the matrix cores are busy.
+// Per 32-key step and wave:
+//   S^T[kv, q]  = K_step . Q^T          4 x RQ v_mfma_f32_32x32x16 (D = 64)
+//   online softmax in the accumulator layout: a lane holds 16 of the 32 scores
+//   of ONE query row, the other 16 sit in lane ^ 32 -> row max/sum are
+//   in-register reductions plus one permlane32 swap; the reference maximum only
+//   moves when it is beaten by 2^8, so the accumulator is rarely rescaled
+//   O^T[d, q] += V_step^T . P^T         4 x RQ v_mfma (P^T is already in B-operand
 //   layout; V^T fragments come from transposing LDS reads)
 #include "mfma_common.cuh"
 
 namespace flex {
 
-constexpr int kFwdBM = 128;
 constexpr int kFwdBN = 64;
+__host__ __device__ constexpr int fwd_rq(int D) { return D == 64 ? 2 : 1; }
+__host__ __device__ constexpr int fwd_bm(int D) { return 4 * 32 * fwd_rq(D); }
 
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(256, D == 64 ? 3 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2) {
   typedef typename Frag<T>::vec8 vec8;
-  constexpr int BM = kFwdBM, BN = kFwdBN;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int RQ = fwd_rq(D), BM = fwd_bm(D), BN = kFwdBN;
   constexpr int DS = D / 16;     // k-steps of the Q.K^T product
   constexpr int DB = D / 32;     // 32-row blocks of O^T
   constexpr int ROWE = D + 8;    // LDS row length in elements (16 B of padding)
   constexpr int CPR = D / 8;     // 16-byte chunks per row
   constexpr int NLD = BN * CPR / 256;  // chunks per thread per tile
-  __shared__ __align__(16) T Ks[BN * ROWE];
-  __shared__ __align__(16) T Vs[BN * ROWE];
+  // two LDS stages: while one tile is consumed the next one is written, so a
+  // single workgroup barrier per tile suffices
+  __shared__ __align__(16) T Ksm[2][BN * ROWE];
+  __shared__ __align__(16) T Vsm[2][BN * ROWE];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
   const int nqt = (p.Lq + BM - 1) / BM;
-  const int total = nqt * p.Hq * p.B;
   int rank, bh;
   xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
   const int qt = nqt - 1 - rank;  // late query tiles see the most keys under causal masks
   const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
 
-  const int q_row = qt * BM + w * 32 + i32;
-  const int q_ld = min(q_row, p.Lq - 1);
+  // this lane's query rows: block a sits at q_row0 + 32 * a
+  const int q_row0 = qt * BM + w * (32 * RQ) + i32;
 
   // Q fragments (B operand of S^T = K.Q^T), resident for the whole kernel
-  vec8 qf[DS];
-  {
+  vec8 qf[RQ][DS];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_ld = min(q_row0 + 32 * a, p.Lq - 1);
     const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
 #pragma unroll
-    for (int s = 0; s < DS; s++) qf[s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+    for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
   }
 
   // tile schedule
@@ -79,27 +90,22 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void fwd_mfma_kernel(FlexAttn
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
-  uint4 kreg[NLD], vreg[NLD];
+  u32x4 kreg[NLD], vreg[NLD];
   auto load_tile = [&](int kv0) {
 #pragma unroll
     for (int j = 0; j < NLD; j++) {
-      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      int kv = kv0 + r;
-      if (kv < p.Lkv) {
-        kreg[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)kv * ks2 + cc * 8);
-        vreg[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)kv * vs2 + cc * 8);
-      } else {
-        kreg[j] = make_uint4(0, 0, 0, 0);
-        vreg[j] = make_uint4(0, 0, 0, 0);
-      }
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
+      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
+      vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int stage) {
 #pragma unroll
     for (int j = 0; j < NLD; j++) {
-      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint4*>(Ks + r * ROWE + cc * 8) = kreg[j];
-      *reinterpret_cast<uint4*>(Vs + r * ROWE + cc * 8) = vreg[j];
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
+      *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
     }
   };
 
@@ -107,118 +113,174 @@ __global__ __launch_bounds__(256, D == 64 ? 3 : 2) void fwd_mfma_kernel(FlexAttn
   sm.init(p.score, p.scale, h);
   Mask2 visible(p.mask, b, h, p.Lkv);
 
-  float16_t oacc[DB];
+  float16_t oacc[RQ][DB];
+  float m_run[RQ], l_run[RQ];
 #pragma unroll
-  for (int db = 0; db < DB; db++)
+  for (int a = 0; a < RQ; a++) {
+    m_run[a] = -INFINITY;
+    l_run[a] = 0.f;
 #pragma unroll
-    for (int r = 0; r < 16; r++) oacc[db][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[a][db][r] = 0.f;
+  }
 
   constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) load_tile(t_cur * BN);
+  // prologue: tile 0 into stage 0, tile 1 into registers
+  if (nt > 0) {
+    load_tile(t_cur * BN);
+    store_tile(0);
+  }
+  if (nt > 1) load_tile(t_nxt * BN);
+  __syncthreads();
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
-    store_tile();
-    __syncthreads();
-    if (it + 1 < nt) load_tile(t_nxt * BN);
+    const T* Ks = Ksm[it & 1];
+    const T* Vs = Vsm[it & 1];
     t_cur = t_nxt;
     if (it + 2 < nt) t_nxt = tile_at(it + 2);
 
-    // Each 32-row half of the tile is one online-softmax step (keeps only 16
-    // score registers live, which is what lets four waves share a SIMD).
+    // Each 32-row half of the tile is one online-softmax step.
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
-      // ---- S^T = K . Q^T ----
-      float16_t sacc;
+      // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
+      vec8 kfr[DS], vfr[2][DB];
+      {
+        const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
 #pragma unroll
-      for (int r = 0; r < 16; r++) sacc[r] = 0.f;
-      const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+        for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
 #pragma unroll
-      for (int s = 0; s < DS; s++) {
-        vec8 a = *reinterpret_cast<const vec8*>(kp + 16 * s);
-        sacc = Frag<T>::mfma(a, qf[s], sacc);
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) {
+            const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+            vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+          }
       }
-
-      // ---- score_mod relative to the running reference max, tile mask where needed ----
-      const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
-      sm.tile(q_row, kv0 + nb * 32 + 4 * g);
+      // ---- S^T = K . Q^T for every query block of the wave ----
+      float16_t sacc[RQ];
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float s0 = sacc[r], s1 = sacc[r + 1];
-        if (ROUND_S) round_pair<T>(s0, s1);
-        sacc[r] = sm.apply_sub(s0, acc_row(r), m_use);
-        sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use);
-      }
-      if (masked) mask_block_q(sacc, p.mask, visible, q_row, kv0 + nb * 32, g, p.Lkv);
+      for (int a = 0; a < RQ; a++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[a][r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < DS; s++)
+#pragma unroll
+        for (int a = 0; a < RQ; a++) sacc[a] = Frag<T>::mfma(kfr[s], qf[a][s], sacc[a]);
 
+      // The query blocks of the wave go through each phase together: their
+      // dependency chains (max tree, lane-half swap, exp) are independent and
+      // interleave, and one branch covers the rare rescale of either block.
+      float m_use[RQ], m_rel[RQ];
+      bool need[RQ], any_need = false;
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        const int q_row = q_row0 + 32 * a;
+        // ---- score_mod relative to the running reference max, tile mask where needed ----
+        m_use[a] = (m_run[a] == -INFINITY) ? 0.f : m_run[a];
+        sm.tile(q_row, kv0 + nb * 32 + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float s0 = sacc[a][r], s1 = sacc[a][r + 1];
+          if (ROUND_S) round_pair<T>(s0, s1);
+          sacc[a][r] = sm.apply_sub(s0, acc_row(r), m_use[a]);
+          sacc[a][r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use[a]);
+        }
+        if (masked) {
+          // a real branch: without the barrier the compiler evaluates the mask for every
+          // tile and selects, which costs as much as the softmax itself
+          // every input of the mask arithmetic passes through this asm, so that none of it
+          // can be hoisted above the branch
+          int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+          asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+          mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+        }
+      }
       // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
-      const float m_rel = xhalf_max(block_max(sacc));
-      const bool need = (m_rel > kTau) || (m_run == -INFINITY && m_rel > -INFINITY);
-      if (__any(need)) {
-        const float delta = need ? m_rel : 0.f;
-        const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(-delta);
-        m_run = need ? (m_use + m_rel) : m_run;
-        l_run *= alpha;
 #pragma unroll
-        for (int r = 0; r < 16; r++) sacc[r] -= delta;
+      for (int a = 0; a < RQ; a++) m_rel[a] = block_max(sacc[a]);
 #pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) oacc[db][r] *= alpha;
+      for (int a = 0; a < RQ; a++) {
+        m_rel[a] = xhalf_max(m_rel[a]);
+        need[a] = (m_rel[a] > kTau) || (m_run[a] == -INFINITY && m_rel[a] > -INFINITY);
+        any_need |= need[a];
       }
-      vec8 pf[2];
+      if (__any(any_need)) {
 #pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        typename Pair<T>::v2 pr[4];
+        for (int a = 0; a < RQ; a++) {
+          float m_opaque = m_rel[a];
+          asm volatile("" : "+v"(m_opaque));  // keeps this rare path a real branch (never if-converted)
+          const float delta = need[a] ? m_opaque : 0.f;
+          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
+          m_run[a] = need[a] ? (m_use[a] + m_rel[a]) : m_run[a];
+          l_run[a] *= alpha;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const float p0 = fast_exp2(sacc[8 * tt + 2 * e]);
-          const float p1 = fast_exp2(sacc[8 * tt + 2 * e + 1]);
-          pr[e] = Pair<T>::pack(p0, p1);
-          l_run = Pair<T>::add_sum(pr[e], l_run);
+          for (int r = 0; r < 16; r++) sacc[a][r] -= delta;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
         }
-        pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
       }
-
-      // ---- O^T += V^T . P^T ----
 #pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
+      for (int a = 0; a < RQ; a++) {
+        vec8 pf[2];
 #pragma unroll
-        for (int db = 0; db < DB; db++) {
-          const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-          short4_t lo = lds_read_tr(vp);
-          short4_t hi = lds_read_tr(vp + 8 * ROWE);
-          oacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), pf[tt], oacc[db]);
+        for (int tt = 0; tt < 2; tt++) {
+          typename Pair<T>::v2 pr[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p0 = fast_exp2(sacc[a][8 * tt + 2 * e]);
+            const float p1 = fast_exp2(sacc[a][8 * tt + 2 * e + 1]);
+            pr[e] = Pair<T>::pack(p0, p1);
+            l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+          }
+          pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
         }
+        // ---- O^T += V^T . P^T (issued before the next block's exponentials so the two overlap) ----
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+      }
+      if (nb == 0 && it + 1 < nt) {
+        // the other stage was last read before the previous barrier: refill it with the
+        // tile prefetched into registers, then start fetching the one after
+        store_tile((it + 1) & 1);
+        if (it + 2 < nt) load_tile(t_nxt * BN);
       }
     }
     __syncthreads();
   }
 
   // ---- epilogue ----
-  const float l_tot = xhalf_sum(l_run);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (q_row < p.Lq) {
-    T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_row * p.o_stride[2] + 4 * g;
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+  for (int a = 0; a < RQ; a++) {
+    const int q_row = q_row0 + 32 * a;
+    const float l_tot = xhalf_sum(l_run[a]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (q_row < p.Lq) {
+      T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_row * p.o_stride[2] + 4 * g;
 #pragma unroll
-      for (int rr = 0; rr < 4; rr++) {
-        union { T e[4]; uint2 u; } pk;
+      for (int db = 0; db < DB; db++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) pk.e[e] = (T)(oacc[db][4 * rr + e] * inv);
-        *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
-      }
-    if (lse2 && g == 0) lse2[((int64_t)b * p.Hq + h) * p.Lq + q_row] = l_tot > 0.f ? m_run + log2f(l_tot) : -INFINITY;
+        for (int rr = 0; rr < 4; rr++) {
+          union { T e[4]; uint2 u; } pk;
+#pragma unroll
+          for (int e = 0; e < 4; e++) pk.e[e] = (T)(oacc[a][db][4 * rr + e] * inv);
+          *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
+        }
+      if (lse2 && g == 0) lse2[((int64_t)b * p.Hq + h) * p.Lq + q_row] = l_tot > 0.f ? m_run[a] + log2f(l_tot) : -INFINITY;
+    }
   }
 }
 
 template <typename T, int D, int KIND>
 static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
-  const int nqt = (p.Lq + kFwdBM - 1) / kFwdBM;
+  const int nqt = (p.Lq + fwd_bm(D) - 1) / fwd_bm(D);
   dim3 grid(nqt * p.Hq * p.B);
   if (p.flags & FLEX_ROUND_S)
     hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
@@ -245,22 +307,26 @@ void flex_set_error(const char* fmt, ...);
 
 static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
 
+// dtype / head size / layout the MFMA kernels can take at all
 bool flex_mfma_shape_ok(const FlexAttnParams& p) {
   if (p.dtype != FLEX_F16 && p.dtype != FLEX_BF16) return false;
   if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
   if (!strides_ok(p.q_stride) || !strides_ok(p.k_stride) || !strides_ok(p.v_stride) || !strides_ok(p.o_stride)) return false;
-  const FlexTileLists& t = p.tiles;
-  if (t.kv_num && (t.q_block != kFwdBM || t.kv_block != kFwdBN)) return false;
-  if ((int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B > 0x7fffffff) return false;
+  if ((int64_t)((p.Lq + 127) / 128) * p.Hq * p.B > 0x7fffffff) return false;
   return true;
 }
 
-bool flex_mfma_fwd_supported(const FlexAttnParams& p) { return flex_mfma_shape_ok(p); }
-
-void flex_mfma_tiles(int dtype, int D, int Dv, int* qb, int* kvb) {
-  bool ok = (dtype == FLEX_F16 || dtype == FLEX_BF16) && D == Dv && (D == 64 || D == 128);
-  *qb = ok ? kFwdBM : 0;
+// which: 0 = forward and decode lists, 1 = backward lists
+void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
+  const bool ok = (dtype == FLEX_F16 || dtype == FLEX_BF16) && D == Dv && (D == 64 || D == 128);
+  *qb = !ok ? 0 : (which == 0 ? fwd_bm(D) : 128);
   *kvb = ok ? kFwdBN : 0;
+}
+
+bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
+  if (!flex_mfma_shape_ok(p)) return false;
+  const FlexTileLists& t = p.tiles;
+  return !t.kv_num || (t.q_block == fwd_bm(p.D) && t.kv_block == kFwdBN);
 }
 
 int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {

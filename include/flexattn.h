@@ -109,16 +109,18 @@ typedef struct FlexAttnParams {
   int32_t flags;
   FlexScoreMod score;
   FlexMask mask;
-  FlexTileLists tiles;
+  FlexTileLists tiles;     /* lists for flexattn_fwd / flexattn_decode */
+  FlexTileLists tiles_bwd; /* lists for flexattn_bwd (its kernels tile differently) */
 } FlexAttnParams;
 
 int flexattn_abi_version(void);
 const char* flexattn_last_error(void);
 
 /* Tile sizes the fused kernels want their FlexTileLists built at for this
- * problem (0/0 when only the generic kernels apply and lists are ignored). */
+ * problem (0/0 when only the generic kernels apply and lists are ignored).
+ * which = 0: FlexAttnParams.tiles (forward, decode); which = 1: tiles_bwd. */
 int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv,
-                             int32_t* q_block, int32_t* kv_block);
+                             int32_t which, int32_t* q_block, int32_t* kv_block);
 
 /* Block-mask builder.  Replaces create_block_mask -> _create_block_mask_inner
  * -> create_mask / _convert_mask_to_block_mask -> _dense_to_ordered

@@ -40,13 +40,13 @@ def test_ctypes_structs_match_c_layout(tmp_path):
     src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "flexattn.h"\n'
                    'int main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(FlexScoreMod), sizeof(FlexMask),'
                    'sizeof(FlexTileLists), sizeof(FlexAttnParams), offsetof(FlexAttnParams, scale),'
-                   'offsetof(FlexAttnParams, score), offsetof(FlexAttnParams, mask), offsetof(FlexAttnParams, tiles));return 0;}\n')
+                   'offsetof(FlexAttnParams, score), offsetof(FlexAttnParams, mask), offsetof(FlexAttnParams, tiles_bwd));return 0;}\n')
     exe = tmp_path / "layout"
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
     got = [int(x) for x in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
     P = _lib.FlexAttnParams
     want = [ctypes.sizeof(_lib.FlexScoreMod), ctypes.sizeof(_lib.FlexMask), ctypes.sizeof(_lib.FlexTileLists),
-            ctypes.sizeof(P), P.scale.offset, P.score.offset, P.mask.offset, P.tiles.offset]
+            ctypes.sizeof(P), P.scale.offset, P.score.offset, P.mask.offset, P.tiles_bwd.offset]
     assert got == want
 
 
@@ -54,9 +54,13 @@ def test_workspace_and_tile_queries_without_gpu():
     L = _lib.lib()
     assert L.flexattn_block_mask_workspace_bytes(2, 3, 4, 5) >= 2 * 2 * 3 * 4 * 5
     qb, kvb = ctypes.c_int32(), ctypes.c_int32()
-    L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, ctypes.byref(qb), ctypes.byref(kvb))
+    L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (256, 64)
+    L.flexattn_preferred_tiles(_lib.FLEX_BF16, 128, 128, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (128, 64)
-    L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, ctypes.byref(qb), ctypes.byref(kvb))
+    L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 1, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (128, 64)
+    L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (0, 0)
     # argument validation happens before anything touches a device
     p = _lib.FlexAttnParams()
