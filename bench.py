@@ -143,16 +143,20 @@ def cpu_baseline(workload):
         dtype, sm, mm, flops, tag = torch.float16, o_checkerboard_kv, None, 240.52e9 / 8, "checkerboard"
     q, k, v = seeded_qkv(1, 8, 8, 2048, 2048, 64, dtype)
     d_o = torch.ones_like(q)
-    t0 = time.perf_counter()
-    ref_attention(q, k, v, sm, mm, strict=True)
-    ref_attention_bwd(q, k, v, d_o, sm, mm, strict=True)
-    dt = time.perf_counter() - t0
-    return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        ref_attention(q, k, v, sm, mm, strict=True)
+        ref_attention_bwd(q, k, v, d_o, sm, mm, strict=True)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt >= 12.0 or reps >= 200:
+            break
+    return {"value": round(flops * reps / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"1 of 8 batch elements of the workload ([1,8,2048,64] {str(dtype).split('.')[-1]}, {tag}), "
-                      f"forward + backward once, {dt:.1f} s"}
+                      f"forward + backward repeated {reps} times, {dt:.1f} s"}
 
 
-def run_train_config(dev, name, steps, warmup, opts=None):
+def make_train_config(dev, name, opts=None):
     from flaxattention_amd.masks import causal_mask
     from flaxattention_amd.mods import generate_alibi_bias, generate_checkerboard
     if name == "config2":
@@ -162,6 +166,11 @@ def run_train_config(dev, name, steps, warmup, opts=None):
     else:
         pr = Prepared(dev, torch.bfloat16, 8, 8, 8, 2048, 2048, 64, generate_alibi_bias(8, -1.0), causal_mask, opts)
         tiles, dtype = 8 * 8 * tiles_128("causal", 2048), "bf16"
+    return pr, tiles, dtype
+
+
+def run_train_config(dev, name, steps, warmup, opts=None):
+    pr, tiles, dtype = make_train_config(dev, name, opts)
     per_tile = 128 * 128 * 64
     f_fwd, f_bwd = 4 * per_tile * tiles, 10 * per_tile * tiles
 
@@ -179,6 +188,23 @@ def run_train_config(dev, name, steps, warmup, opts=None):
     return {"ms_per_step": ms, "tflops": (f_fwd + f_bwd) / ms / 1e9, "fwd_tflops": f_fwd / us["fwd_mfma_kernel"] / 1e6,
             "bwd_tflops": f_bwd / (us["bwd_dq_kernel"] + us["bwd_dkv_kernel"]) / 1e6,
             "kernels": kern, "dominant": dom, "dtype": dtype, "flops": f_fwd + f_bwd}
+
+
+def pmc_probe(dev, name, opts):
+    """What a hardware-counter run should see: a device-to-device copy of known size (1 GiB read, 1 GiB written)
+    to calibrate the byte counters against, then each kernel of the workload three times."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    pr = make_train_config(dev, name, opts)[0]
+    for _ in range(3):
+        pr.fwd()
+        pr.bwd("dq")
+        pr.bwd("dkv")
+    torch.cuda.synchronize()
 
 
 def run_config4(dev, steps, warmup):
@@ -223,6 +249,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all", action="store_true", help="also run configurations 3, 4 and 5 (reported on stderr and in 'extra')")
     ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="counter run: one 1 GiB device copy (calibration) and 3 launches of each kernel of the workload, nothing else")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (attention shards over batch x head "
@@ -233,6 +261,9 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda", 0)
     opts = {"round_s": bool(a.round_s)}
+    if a.pmc_probe:
+        pmc_probe(dev, a.workload, opts)
+        return
     r = run_train_config(dev, a.workload, a.steps, a.warmup, opts)
     log(f"{a.workload}: {r['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r['tflops']:.1f} TFLOP/s  "
         f"(fwd {r['fwd_tflops']:.1f}, bwd {r['bwd_tflops']:.1f})  kernels {r['kernels']}")

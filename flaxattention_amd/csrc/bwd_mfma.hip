@@ -25,7 +25,7 @@ constexpr int kBM = 128;  // query tile (list granularity)
 constexpr int kBN = 64;   // key tile (list granularity)
 
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(256) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
                                                       const T* __restrict__ d_o, T* __restrict__ dq,

@@ -278,10 +278,288 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   }
 }
 
+// ---------------------------------------------------------------------------
+// D = 64: software-pipelined variant.  A wave owns two blocks of 32 query rows
+// and walks "units" (32-key step, query block).  The instruction stream of a
+// unit pairs every group of matrix instructions with independent vector work,
+// so that the matrix pipe and the vector ALU of a SIMD run at the same time
+// even when the waves of a workgroup march in lockstep:
+//   region A: scale / score_mod of S(u)            ||  S^T = K.Q^T of unit u+1
+//   (tile mask if needed, row max, rare rescale of the accumulator)
+//   region B: exponentials, rounding, row sum      ||  O^T += V^T.P^T of unit u-1
+// Every matrix result is first read at least half a unit after it was issued.
+// Unit u-1 and unit u+1 belong to the wave's other query block, so a rescale in
+// unit u never touches an accumulator that a matrix instruction is writing.
+// KV tiles go through three LDS stages with one workgroup barrier per tile: a
+// stage is refilled only after a barrier that follows its last fragment read.
+// ---------------------------------------------------------------------------
+template <typename T, int KIND, bool ROUND_S>
+__global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                           const T* __restrict__ k, const T* __restrict__ v,
+                                                           T* __restrict__ o, float* __restrict__ lse2) {
+  typedef typename Frag<T>::vec8 vec8;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int D = 64, RQ = 2, BM = fwd_bm(D), BN = kFwdBN;
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
+  static_assert(fwd_rq(D) == RQ, "two query blocks per wave");
+  __shared__ __align__(16) T Ksm[3][BN * ROWE];
+  __shared__ __align__(16) T Vsm[3][BN * ROWE];
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
+  const int nqt = (p.Lq + BM - 1) / BM;
+  int rank, bh;
+  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
+  const int qt = nqt - 1 - rank;
+  const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int q_row0 = qt * BM + w * (32 * RQ) + i32;
+
+  vec8 qf[RQ][DS];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_ld = min(q_row0 + 32 * a, p.Lq - 1);
+    const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+  }
+
+  const FlexTileLists& tl = p.tiles;
+  const int32_t* full_idx = nullptr;
+  const int32_t* part_idx = nullptr;
+  int n_full, n_part = 0;
+  if (tl.kv_num) {
+    const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
+    n_full = tl.full_kv_num[row];
+    n_part = tl.kv_num[row];
+    full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
+    part_idx = tl.kv_idx + row * tl.n_kv_blocks;
+  } else {
+    n_full = (p.Lkv + BN - 1) / BN;
+  }
+  const int nt = n_full + n_part;
+  auto tile_at = [&](int it) -> int {
+    if (!full_idx) return it;
+    return it < n_full ? full_idx[it] : part_idx[it - n_full];
+  };
+
+  const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
+  const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
+  const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
+
+  u32x4 kreg[NLD], vreg[NLD];
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      const int kvc = min(kv0 + r, p.Lkv - 1);
+      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
+      vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+    }
+  };
+  auto store_tile = [&](int stage) {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
+      *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
+    }
+  };
+  vec8 kfr[DS], vfr[2][DB], pf[2];
+  auto read_k = [&](const T* Ks, int nb) {
+    const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+  };
+  auto read_v = [&](const T* Vs, int nb) {
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+        vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+      }
+  };
+
+  Score2<KIND> sm;
+  sm.init(p.score, p.scale, h);
+  Mask2 visible(p.mask, b, h, p.Lkv);
+
+  float16_t oacc[RQ][DB], s_cur;
+  float m_run[RQ], l_run[RQ];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    m_run[a] = -INFINITY;
+    l_run[a] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[a][db][r] = 0.f;
+  }
+  // nothing is pending before the first unit: P = 0 against V = 0
+#pragma unroll
+  for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) pf[tt][e] = (T)0.f;
+#pragma unroll
+    for (int db = 0; db < DB; db++) vfr[tt][db] = pf[tt];
+  }
+
+  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  int t_cur = nt > 0 ? tile_at(0) : 0;
+  int t_nxt = nt > 1 ? tile_at(1) : 0;
+  if (nt > 0) {
+    load_tile(t_cur * BN);
+    store_tile(0);
+  }
+  if (nt > 1) load_tile(t_nxt * BN);
+  __syncthreads();
+  // S of the first unit
+  read_k(Ksm[0], 0);
+#pragma unroll
+  for (int r = 0; r < 16; r++) s_cur[r] = 0.f;
+#pragma unroll
+  for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
+
+  int st = 0;  // LDS stage of the current tile (it % 3)
+  for (int it = 0; it < nt; it++) {
+    const int kv0 = t_cur * BN;
+    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
+    const int st_n = st == 2 ? 0 : st + 1;
+    const T* Ks = Ksm[st];
+    const T* Vs = Vsm[st];
+    const T* Kn = Ksm[st_n];
+    t_cur = t_nxt;
+    if (it + 2 < nt) t_nxt = tile_at(it + 2);
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        const int q_row = q_row0 + 32 * a;
+        if (nb == 0 && a == 1 && it + 1 < nt) {
+          // stage st_n held the tile before the previous one; its last reads came before the
+          // previous barrier.  Refill it from the prefetch registers and fetch the tile after.
+          store_tile(st_n);
+          if (it + 2 < nt) load_tile(t_nxt * BN);
+        }
+        if (nb == 1 && a == 0) __syncthreads();  // the next tile's stage is complete
+        if (a == 1) read_v(Vs, nb);              // V columns of this step, first used in region B
+
+        // ---- region A: S^T of the next unit || score_mod relative to the running reference max ----
+        float16_t s_nxt;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s_nxt[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; s++) s_nxt = Frag<T>::mfma(kfr[s], qf[1 - a][s], s_nxt);
+        const float m_use = (m_run[a] == -INFINITY) ? 0.f : m_run[a];
+        sm.tile(q_row, kv0 + nb * 32 + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float s0 = s_cur[r], s1 = s_cur[r + 1];
+          if (ROUND_S) round_pair<T>(s0, s1);
+          s_cur[r] = sm.apply_sub(s0, acc_row(r), m_use);
+          s_cur[r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use);
+        }
+#pragma unroll
+        for (int i = 0; i < DS; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one matrix instruction
+          if (a == 1) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads (V columns)
+          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // six vector instructions
+        }
+        if (masked) {
+          // a real branch whose inputs pass through the asm, so that none of the mask
+          // arithmetic can be hoisted into the unmasked path
+          int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+          asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+          mask_block_q(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+        }
+        // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
+        float m_rel = xhalf_max(block_max(s_cur));
+        const bool need = (m_rel > kTau) || (m_run[a] == -INFINITY && m_rel > -INFINITY);
+        if (__any(need)) {
+          asm volatile("" : "+v"(m_rel));  // keeps this rare path a real branch (never if-converted)
+          const float delta = need ? m_rel : 0.f;
+          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
+          m_run[a] = need ? (m_use + m_rel) : m_run[a];
+          l_run[a] *= alpha;
+#pragma unroll
+          for (int r = 0; r < 16; r++) s_cur[r] -= delta;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
+        }
+        // ---- region B: O^T += V^T.P^T of the previous unit || exponentials, rounding, row sum ----
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) oacc[1 - a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[1 - a][db]);
+        vec8 pn[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+          typename Pair<T>::v2 pr[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p0 = fast_exp2(s_cur[8 * tt + 2 * e]);
+            const float p1 = fast_exp2(s_cur[8 * tt + 2 * e + 1]);
+            pr[e] = Pair<T>::pack(p0, p1);
+            l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+          }
+          pn[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        }
+        if (a == 0) read_k(nb == 0 ? Ks : Kn, nb == 0 ? 1 : 0);  // K rows of the next step (kfr is free after region A)
+#pragma unroll
+        for (int i = 0; i < 2 * DB; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one matrix instruction
+          if (a == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read (K rows)
+          __builtin_amdgcn_sched_group_barrier(0x400, 4, 0);             // four exponentials
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // rounding and row sum of the previous four
+        }
+        pf[0] = pn[0];
+        pf[1] = pn[1];
+        s_cur = s_nxt;
+      }
+    }
+    st = st_n;
+  }
+  // the last unit's P is still pending
+#pragma unroll
+  for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+    for (int db = 0; db < DB; db++) oacc[1][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[1][db]);
+
+  // ---- epilogue ----
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_row = q_row0 + 32 * a;
+    const float l_tot = xhalf_sum(l_run[a]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (q_row < p.Lq) {
+      T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_row * p.o_stride[2] + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+          union { T e[4]; uint2 u; } pk;
+#pragma unroll
+          for (int e = 0; e < 4; e++) pk.e[e] = (T)(oacc[a][db][4 * rr + e] * inv);
+          *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
+        }
+      if (lse2 && g == 0) lse2[((int64_t)b * p.Hq + h) * p.Lq + q_row] = l_tot > 0.f ? m_run[a] + log2f(l_tot) : -INFINITY;
+    }
+  }
+}
+
 template <typename T, int D, int KIND>
 static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
   const int nqt = (p.Lq + fwd_bm(D) - 1) / fwd_bm(D);
   dim3 grid(nqt * p.Hq * p.B);
+  if constexpr (D == 64) {
+    if (p.flags & FLEX_ROUND_S)
+      hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+    else
+      hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+    return;
+  }
   if (p.flags & FLEX_ROUND_S)
     hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
   else
