@@ -33,13 +33,14 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
   typedef typename Frag<T>::vec8 vec8;
   constexpr int BM = kBM, BN = kBN;
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
-  __shared__ __align__(16) T Ks[BN * ROWE];
-  __shared__ __align__(16) T Vs[BN * ROWE];
+  // two LDS stages: while one tile is consumed the next one is written, so a
+  // single workgroup barrier per tile suffices
+  __shared__ __align__(16) T Ksm[2][BN * ROWE];
+  __shared__ __align__(16) T Vsm[2][BN * ROWE];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
   const int nqt = (p.Lq + BM - 1) / BM;
-  const int total = nqt * p.Hq * p.B;
   int rank, bh;
   xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
   const int qt = nqt - 1 - rank;
@@ -90,27 +91,23 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
-  uint4 kreg[NLD], vreg[NLD];
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  u32x4 kreg[NLD], vreg[NLD];
   auto load_tile = [&](int kv0) {
 #pragma unroll
     for (int j = 0; j < NLD; j++) {
-      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      int kv = kv0 + r;
-      if (kv < p.Lkv) {
-        kreg[j] = *reinterpret_cast<const uint4*>(kbase + (int64_t)kv * ks2 + cc * 8);
-        vreg[j] = *reinterpret_cast<const uint4*>(vbase + (int64_t)kv * vs2 + cc * 8);
-      } else {
-        kreg[j] = make_uint4(0, 0, 0, 0);
-        vreg[j] = make_uint4(0, 0, 0, 0);
-      }
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
+      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
+      vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int stage) {
 #pragma unroll
     for (int j = 0; j < NLD; j++) {
       int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<uint4*>(Ks + r * ROWE + cc * 8) = kreg[j];
-      *reinterpret_cast<uint4*>(Vs + r * ROWE + cc * 8) = vreg[j];
+      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
+      *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
     }
   };
 
@@ -125,21 +122,35 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
 
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) load_tile(t_cur * BN);
+  if (nt > 0) {
+    load_tile(t_cur * BN);
+    store_tile(0);
+  }
+  if (nt > 1) load_tile(t_nxt * BN);
+  __syncthreads();
+  const float neg_delta = -delta;
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
-    store_tile();
-    __syncthreads();
-    if (it + 1 < nt) load_tile(t_nxt * BN);
-    t_cur = t_nxt;
-    if (it + 2 < nt) t_nxt = tile_at(it + 2);
+    const T* Ks = Ksm[it & 1];
+    const T* Vs = Vsm[it & 1];
+    if (it + 1 < nt) {
+      // the other stage was last read before the previous barrier: refill it with the
+      // tile prefetched into registers, then start fetching the one after
+      store_tile((it + 1) & 1);
+      t_cur = t_nxt;
+      if (it + 2 < nt) {
+        t_nxt = tile_at(it + 2);
+        load_tile(t_nxt * BN);
+      }
+    }
 
+    // dP starts at -delta, so the accumulator comes out as dP - delta
     float16_t sacc[2], dpacc[2];
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
-      for (int r = 0; r < 16; r++) { sacc[nb][r] = 0.f; dpacc[nb][r] = 0.f; }
+      for (int r = 0; r < 16; r++) { sacc[nb][r] = 0.f; dpacc[nb][r] = neg_delta; }
       const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
       const T* vp = Vs + (nb * 32 + i32) * ROWE + 8 * g;
 #pragma unroll
@@ -175,8 +186,8 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 8 * tt + 2 * e;
-          float d0 = fast_exp2(sacc[nb][r]) * (dpacc[nb][r] - delta);
-          float d1 = fast_exp2(sacc[nb][r + 1]) * (dpacc[nb][r + 1] - delta);
+          float d0 = fast_exp2(sacc[nb][r]) * dpacc[nb][r];
+          float d1 = fast_exp2(sacc[nb][r + 1]) * dpacc[nb][r + 1];
           if (!Score2<KIND>::kGradOne) { d0 *= gacc[nb][r]; d1 *= gacc[nb][r + 1]; }
           pr[e] = Pair<T>::pack(d0, d1);
         }
@@ -221,6 +232,7 @@ template <int D> struct DkvShape {
   static constexpr int kThreads = kWaves * 64;
   static constexpr int kNQG = kWaves / 2;        // query groups
   static constexpr int kQBlocks = 4 / kNQG;      // 32-row query blocks per wave and tile
+  static constexpr int kStages = D == 64 ? 2 : 1;  // LDS stages of the query-side tiles
 };
 
 template <typename T, int D, int KIND, bool ROUND_S>
@@ -235,10 +247,12 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
   constexpr int BM = kBM, BN = kBN;
   constexpr int kDkvThreads = DkvShape<D>::kThreads, NQG = DkvShape<D>::kNQG, QBW = DkvShape<D>::kQBlocks;
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
-  T* Qs = reinterpret_cast<T*>(bwd_smem);
-  T* Os = Qs + BM * ROWE;
-  float* lse_s = reinterpret_cast<float*>(Os + BM * ROWE);
-  float* del_s = lse_s + BM;
+  // LDS stages of (Q tile, dO tile, lse, -delta).  D = 64 keeps two, so that one workgroup
+  // barrier per tile suffices; with D = 128 a second stage would cost the second workgroup
+  // of the compute unit, so one stage is refilled between two barriers.
+  constexpr int NSTG = DkvShape<D>::kStages;
+  constexpr int kStageBytes = 2 * BM * ROWE * (int)sizeof(T) + 2 * BM * (int)sizeof(float);
+  auto stage_q = [&](int st) { return reinterpret_cast<T*>(bwd_smem + st * kStageBytes); };
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -313,33 +327,67 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
     };
     int t_cur = nt > 0 ? tile_at(0) : 0;
     int t_nxt = nt > 1 ? tile_at(1) : 0;
-    if (nt > 0) load_tile(t_cur * BM);
-    for (int it = 0; it < nt; it++) {
-      const int q0 = t_cur * BM;
-      const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
-      __syncthreads();  // previous tile fully consumed
+    auto store_tile = [&](int st) {
+      T* Qw = stage_q(st);
+      T* Ow = Qw + BM * ROWE;
+      float* lw = reinterpret_cast<float*>(Ow + BM * ROWE);
 #pragma unroll
       for (int j = 0; j < NLD; j++) {
         const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
-        *reinterpret_cast<u32x4*>(Qs + r * ROWE + cc * 8) = qreg[j];
-        *reinterpret_cast<u32x4*>(Os + r * ROWE + cc * 8) = oreg[j];
+        *reinterpret_cast<u32x4*>(Qw + r * ROWE + cc * 8) = qreg[j];
+        *reinterpret_cast<u32x4*>(Ow + r * ROWE + cc * 8) = oreg[j];
       }
       if (tid < BM) {
-        lse_s[tid] = lreg;   // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
-        del_s[tid] = dreg;
+        lw[tid] = lreg;        // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
+        lw[BM + tid] = -dreg;  // the dP accumulator starts from -delta
       }
+    };
+    __syncthreads();  // the stages may still be in use by the previous head of the group
+    if (nt > 0) load_tile(t_cur * BM);
+    if (NSTG == 2) {
+      if (nt > 0) store_tile(0);
+      if (nt > 1) load_tile(t_nxt * BM);
       __syncthreads();
-      if (it + 1 < nt) load_tile(t_nxt * BM);
-      t_cur = t_nxt;
-      if (it + 2 < nt) t_nxt = tile_at(it + 2);
+    }
+    for (int it = 0; it < nt; it++) {
+      const int q0 = t_cur * BM;
+      const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
+      const int st = NSTG == 2 ? (it & 1) : 0;
+      const T* Qs = stage_q(st);
+      const T* Os = Qs + BM * ROWE;
+      const float* lse_s = reinterpret_cast<const float*>(Os + BM * ROWE);
+      const float* del_s = lse_s + BM;
+      if (NSTG == 2) {
+        if (it + 1 < nt) {
+          // the other stage was last read before the previous barrier: refill it with the
+          // tile prefetched into registers, then start fetching the one after
+          store_tile((it + 1) & 1);
+          t_cur = t_nxt;
+          if (it + 2 < nt) {
+            t_nxt = tile_at(it + 2);
+            load_tile(t_nxt * BM);
+          }
+        }
+      } else {
+        store_tile(0);  // the barrier that closed the previous tile freed the stage
+        __syncthreads();
+        if (it + 1 < nt) load_tile(t_nxt * BM);
+        t_cur = t_nxt;
+        if (it + 2 < nt) t_nxt = tile_at(it + 2);
+      }
 
 #pragma unroll
       for (int qs = 0; qs < QBW; qs++) {
       // ---- S = Q.K^T and dP = dO.V^T for 32 query rows x 32 keys ----
       const int qrow_w = (wq * QBW + qs) * 32;
       float16_t sacc, dpacc;
+      const int ql = qrow_w + 4 * g;  // local row of register 0
 #pragma unroll
-      for (int r = 0; r < 16; r++) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+      for (int rr = 0; rr < 4; rr++) {
+        const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
+#pragma unroll
+        for (int e = 0; e < 4; e++) { sacc[4 * rr + e] = 0.f; dpacc[4 * rr + e] = d4[e]; }
+      }
       {
         const T* qp = Qs + (qrow_w + i32) * ROWE + 8 * g;
         const T* op = Os + (qrow_w + i32) * ROWE + 8 * g;
@@ -351,12 +399,10 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
       }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
       float16_t gacc;
-      const int ql = qrow_w + 4 * g;  // local row of register 0
       sm.tileT(q0 + ql, kv_col);
 #pragma unroll
       for (int rr = 0; rr < 4; rr++) {
         const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
-        const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
           const int r = 4 * rr + e;
@@ -364,8 +410,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
           if (ROUND_S) round_pair<T>(s0, s1);
           sacc[r] = sm.apply_sub(s0, acc_row(r), l4[e]);
           sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), l4[e + 1]);
-          dpacc[r] -= d4[e];
-          dpacc[r + 1] -= d4[e + 1];
           if (!Score2<KIND>::kGradOne) {
             gacc[r] = sm.grad(s0, acc_row(r));
             gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
@@ -402,6 +446,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
         }
       }
       }  // query blocks of this wave
+      __syncthreads();
     }
   }
 
@@ -457,7 +502,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
 }
 
 template <int D, typename T> constexpr size_t dkv_smem() {
-  size_t tiles = (size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float);
+  size_t tiles = DkvShape<D>::kStages * ((size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
   size_t red = (size_t)2 * 2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
   return tiles > red ? tiles : red;
 }
