@@ -13,10 +13,9 @@
 //  bwd_dkv_kernel  one workgroup per 64 key rows, sweeping query tiles of 128
 //                  from the transposed tile lists.  Here a lane owns one key
 //                  row: S = Q.K^T, dP = dO.V^T, dV^T += dO^T.P, dK^T += Q^T.dS.
-//                  Eight waves = 2 key blocks x 4 query quarters (two waves per
-//                  SIMD, so one wave's MFMA overlaps the other's vector work);
-//                  the quarters are summed through LDS at the end.  With GQA the workgroup loops over the query
-//                  heads of its group.
+//                  Four waves = 2 key blocks x 2 query halves; the halves are
+//                  summed through LDS at the end.  With GQA the workgroup loops
+//                  over the query heads of its group.
 #include "mfma_common.cuh"
 
 namespace flex {
@@ -223,12 +222,12 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
 
 extern __shared__ __align__(16) unsigned char bwd_smem[];
 
-// dK/dV workgroup: 2 key blocks x NQG query groups.  D = 64 runs 8 waves (two per
-// SIMD, so one wave's MFMA overlaps the other's vector work); D = 128 needs the
-// registers of a full SIMD per wave and runs 4 waves, each taking two 32-row
-// query blocks in turn.
+// dK/dV workgroup: 4 waves = 2 key blocks x 2 query groups, each wave taking two
+// 32-row query blocks of a tile in turn.  With D = 64 two such workgroups share a
+// compute unit (two waves per SIMD); being independent they drift out of phase,
+// so one's matrix work overlaps the other's vector work and barrier waits.
 template <int D> struct DkvShape {
-  static constexpr int kWaves = D == 64 ? 8 : 4;
+  static constexpr int kWaves = 4;
   static constexpr int kThreads = kWaves * 64;
   static constexpr int kNQG = kWaves / 2;        // query groups
   static constexpr int kQBlocks = 4 / kNQG;      // 32-row query blocks per wave and tile
@@ -236,7 +235,7 @@ template <int D> struct DkvShape {
 };
 
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                                const T* __restrict__ k, const T* __restrict__ v,
                                                                const float* __restrict__ lse2,
                                                                const float* __restrict__ delta,
@@ -282,6 +281,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
 
   const FlexTileLists& tl = p.tiles_bwd;
   Score2<KIND> sm;
+  float key_grad = 1.f;  // derivative of a score_mod that depends on the key only: applied to dK at the end
 
   for (int gi = 0; gi < G; gi++) {
     const int h = hk * G + gi;
@@ -400,6 +400,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
       float16_t gacc;
       sm.tileT(q0 + ql, kv_col);
+      if constexpr (KIND == kScoreCheckerboardKv) key_grad = sm.key_grad;
 #pragma unroll
       for (int rr = 0; rr < 4; rr++) {
         const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
@@ -492,7 +493,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads) void bwd_dkv_kernel(FlexAttn
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 4 * rr + e;
-          pk.e[e] = (T)(dkacc[db][r] * p.scale);  // the scale factor of dS is applied once here
+          pk.e[e] = (T)(dkacc[db][r] * (p.scale * key_grad));  // the scale factor of dS is applied once here
           pv.e[e] = (T)dvacc[db][r];
         }
         *reinterpret_cast<uint2*>(dkp + 32 * db + 8 * rr) = pk.u;
@@ -522,6 +523,20 @@ static int launch_one(const FlexAttnParams& p, const void* q, const void* k, con
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
     if (e != hipSuccess) return 2;
     attr_set = true;
+  }
+  if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.i0) {
+    // keyed on the key index: the derivative is constant along a lane's dK row
+    constexpr int KV = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardKv : KIND;
+    static bool attr_kv = false;
+    if (!attr_kv) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KV, RS>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
+      if (e != hipSuccess) return 2;
+      attr_kv = true;
+    }
+    hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KV, RS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p, (const T*)q,
+                       (const T*)k, (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
+    return 0;
   }
   hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p, (const T*)q, (const T*)k,
                      (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);

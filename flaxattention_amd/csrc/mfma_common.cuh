@@ -108,6 +108,24 @@ template <> struct Score2<FLEX_SCORE_CHECKERBOARD> {
   __device__ __forceinline__ float grad(float s, int off) const { return (off & 1) ? fo : fe; }
 };
 
+// Checkerboard keyed on the key index alone, for kernels in which a lane owns one key
+// (dK/dV): factor and derivative are per-lane constants, so the derivative leaves the
+// inner loop and scales the lane's dK row once at the end (key_grad).
+constexpr int kScoreCheckerboardKv = 100;
+template <> struct Score2<kScoreCheckerboardKv> {
+  static constexpr bool kGradOne = true;  // inside the loop; see key_grad
+  float c0, c1, f0, f1, ck, key_grad;
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+    f0 = m.p0; f1 = m.p1; c0 = m.p0 * scale * kLog2e; c1 = m.p1 * scale * kLog2e;
+  }
+  __device__ __forceinline__ void tileT(int qb, int kv) {
+    ck = (kv & 1) ? c1 : c0;
+    key_grad = (kv & 1) ? f1 : f0;
+  }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, ck, -m); }
+  __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
+};
+
 template <> struct Score2<FLEX_SCORE_ALIBI> {
   static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;
