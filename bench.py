@@ -179,13 +179,13 @@ def run_train_config(dev, name, steps, warmup, opts=None):
         pr.bwd()
     ms = wall_time_ms(step, steps, warmup)
     n = max(steps, 10)
-    us = {"fwd_mfma_kernel": event_time_us(pr.fwd, n),
+    us = {"fwd_pipe_kernel": event_time_us(pr.fwd, n),
           "bwd_dq_kernel": event_time_us(lambda: pr.bwd("dq"), n),
           "bwd_dkv_kernel": event_time_us(lambda: pr.bwd("dkv"), n)}
-    alg = {"fwd_mfma_kernel": f_fwd, "bwd_dq_kernel": 2 * per_tile * tiles, "bwd_dkv_kernel": 8 * per_tile * tiles}
+    alg = {"fwd_pipe_kernel": f_fwd, "bwd_dq_kernel": 2 * per_tile * tiles, "bwd_dkv_kernel": 8 * per_tile * tiles}
     kern = {k: {"us": round(us[k], 2), "algorithmic_flops": alg[k], "tflops": round(alg[k] / us[k] / 1e6, 1)} for k in us}
     dom = max(us, key=us.get)
-    return {"ms_per_step": ms, "tflops": (f_fwd + f_bwd) / ms / 1e9, "fwd_tflops": f_fwd / us["fwd_mfma_kernel"] / 1e6,
+    return {"ms_per_step": ms, "tflops": (f_fwd + f_bwd) / ms / 1e9, "fwd_tflops": f_fwd / us["fwd_pipe_kernel"] / 1e6,
             "bwd_tflops": f_bwd / (us["bwd_dq_kernel"] + us["bwd_dkv_kernel"]) / 1e6,
             "kernels": kern, "dominant": dom, "dtype": dtype, "flops": f_fwd + f_bwd}
 

@@ -144,62 +144,64 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
       }
     }
 
-    // dP starts at -delta, so the accumulator comes out as dP - delta
-    float16_t sacc[2], dpacc[2];
+    // one 32-key block at a time (S, dP, softmax, dQ): half the accumulator registers of
+    // doing both blocks side by side
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
+      // dP starts at -delta, so the accumulator comes out as dP - delta
+      float16_t sacc, dpacc, gacc;
 #pragma unroll
-      for (int r = 0; r < 16; r++) { sacc[nb][r] = 0.f; dpacc[nb][r] = neg_delta; }
+      for (int r = 0; r < 16; r++) { sacc[r] = 0.f; dpacc[r] = neg_delta; }
       const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
       const T* vp = Vs + (nb * 32 + i32) * ROWE + 8 * g;
 #pragma unroll
       for (int s = 0; s < DS; s++) {
-        sacc[nb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + 16 * s), qf[s], sacc[nb]);
-        dpacc[nb] = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + 16 * s), dof[s], dpacc[nb]);
+        sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + 16 * s), qf[s], sacc);
+        dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + 16 * s), dof[s], dpacc);
       }
-    }
-    // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
-    float16_t gacc[2];
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+      // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
       sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
-        float s0 = sacc[nb][r], s1 = sacc[nb][r + 1];
+        float s0 = sacc[r], s1 = sacc[r + 1];
         if (ROUND_S) round_pair<T>(s0, s1);
-        sacc[nb][r] = sm.apply_sub(s0, acc_row(r), lse);
-        sacc[nb][r + 1] = sm.apply_sub(s1, acc_row(r + 1), lse);
+        sacc[r] = sm.apply_sub(s0, acc_row(r), lse);
+        sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), lse);
         if (!Score2<KIND>::kGradOne) {
-          gacc[nb][r] = sm.grad(s0, acc_row(r));
-          gacc[nb][r + 1] = sm.grad(s1, acc_row(r + 1));
+          gacc[r] = sm.grad(s0, acc_row(r));
+          gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
         }
       }
-    }
-    if (masked) mask_tile_q(sacc, p.mask, visible, q_row, kv0, g, p.Lkv);
-    vec8 dsf[4];
-#pragma unroll
-    for (int nb = 0; nb < 2; nb++)
+      if (masked) {
+        // a real branch whose inputs pass through the asm, so that none of the mask
+        // arithmetic can be hoisted into the unmasked path
+        int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+        asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+        mask_block_q(sacc, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+      }
+      vec8 dsf[2];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
         typename Pair<T>::v2 pr[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 8 * tt + 2 * e;
-          float d0 = fast_exp2(sacc[nb][r]) * dpacc[nb][r];
-          float d1 = fast_exp2(sacc[nb][r + 1]) * dpacc[nb][r + 1];
-          if (!Score2<KIND>::kGradOne) { d0 *= gacc[nb][r]; d1 *= gacc[nb][r + 1]; }
+          float d0 = fast_exp2(sacc[r]) * dpacc[r];
+          float d1 = fast_exp2(sacc[r + 1]) * dpacc[r + 1];
+          if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
           pr[e] = Pair<T>::pack(d0, d1);
         }
-        dsf[2 * nb + tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        dsf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
       }
 #pragma unroll
-    for (int t = 0; t < 4; t++) {
+      for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
-      for (int db = 0; db < DB; db++) {
-        const T* kp = Ks + (16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-        short4_t lo = lds_read_tr(kp);
-        short4_t hi = lds_read_tr(kp + 8 * ROWE);
-        dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[t], dqacc[db]);
+        for (int db = 0; db < DB; db++) {
+          const T* ktp = Ks + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+          short4_t lo = lds_read_tr(ktp);
+          short4_t hi = lds_read_tr(ktp + 8 * ROWE);
+          dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[tt], dqacc[db]);
+        }
       }
     }
     __syncthreads();
