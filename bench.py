@@ -33,6 +33,16 @@ PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 PEAK_HBM_GBPS = 8000.0
 
 
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE from two `rocprofv3 --pmc` runs of `bench.py --pmc-probe`, each
+# counter scaled by what it reads for a 1 GiB device copy: x2.000 and x1.000); the summary of those runs is kept
+# under profiles/.  Keyed by (workload, kernel); a kernel that has not been measured reports null.
+MEASURED_TRAFFIC_BYTES = {
+    ("config2", "fwd_pipe_kernel"): 67911841,
+    ("config2", "bwd_dq_kernel"): 136536246,
+    ("config2", "bwd_dkv_kernel"): 208139736,
+}
+
+
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
@@ -297,7 +307,8 @@ def main():
         "fwd_tflops": round(r["fwd_tflops"], 1), "bwd_tflops": round(r["bwd_tflops"], 1),
         "kernels": r["kernels"],
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": kd["tflops"], "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(kd["tflops"] / PEAK_MFMA_TFLOPS, 4), "traffic": None},
+                     "frac": round(kd["tflops"] / PEAK_MFMA_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom))},
     }
     if extra:
         line["extra"] = extra
