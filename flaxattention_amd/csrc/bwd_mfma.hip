@@ -5,23 +5,23 @@
 // path.  P is recomputed from the saved base-2 log-sum-exp.  Two kernels:
 //
 //  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 64
-//                  (the forward's schedule).  Transposed products keep one query
+//                  (two per entry of the 128-granular backward lists).  Transposed products keep one query
 //                  row per lane, so lse and delta are per-lane scalars:
 //                    S^T = K.Q^T,  dP^T = V.dO^T,  dS^T = P^T o (dP^T - delta) * g,
 //                    dQ^T += K^T.dS^T.
 //                  Also produces delta_i = sum_d O_id dO_id for the second kernel.
-//  bwd_dkv_kernel  one workgroup per 64 key rows, sweeping query tiles of 128
+//  bwd_dkv_kernel  one workgroup per 128 key rows, sweeping query tiles of 128
 //                  from the transposed tile lists.  Here a lane owns one key
 //                  row: S = Q.K^T, dP = dO.V^T, dV^T += dO^T.P, dK^T += Q^T.dS.
-//                  Four waves = 2 key blocks x 2 query halves; the halves are
-//                  summed through LDS at the end.  With GQA the workgroup loops
-//                  over the query heads of its group.
+//                  Four waves = four key blocks of 32 rows.  With GQA the
+//                  workgroup loops over the query heads of its group.
 #include "mfma_common.cuh"
 
 namespace flex {
 
-constexpr int kBM = 128;  // query tile (list granularity)
-constexpr int kBN = 64;   // key tile (list granularity)
+constexpr int kBM = 128;     // query tile (list granularity)
+constexpr int kBN = 64;      // key tile staged per step by the dQ kernel
+constexpr int kListBN = 128; // key granularity of the backward tile lists = key rows of a dK/dV workgroup
 
 template <typename T, int D, int KIND, bool ROUND_S>
 __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
@@ -81,10 +81,15 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
   } else {
     n_full = (p.Lkv + BN - 1) / BN;
   }
-  const int nt = n_full + n_part;
+  // a list entry covers `sub` staged tiles of BN keys (the lists are kListBN-granular);
+  // the schedule below runs over (entry, part) pairs flattened into one index
+  const int sub = full_idx ? tl.kv_block / BN : 1;
+  const int nt = (n_full + n_part) * sub;
+  const int n_full_t = n_full * sub;
   auto tile_at = [&](int it) -> int {
     if (!full_idx) return it;
-    return it < n_full ? full_idx[it] : part_idx[it - n_full];
+    const int e = sub == 2 ? (it >> 1) : it, part = sub == 2 ? (it & 1) : 0;
+    return (e < n_full ? full_idx[e] : part_idx[e - n_full]) * sub + part;
   };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
@@ -130,7 +135,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
   const float neg_delta = -delta;
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
-    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
+    const bool masked = (it >= n_full_t) || (kv0 + BN > p.Lkv);
     const T* Ks = Ksm[it & 1];
     const T* Vs = Vsm[it & 1];
     if (it + 1 < nt) {
@@ -224,15 +229,15 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
 
 extern __shared__ __align__(16) unsigned char bwd_smem[];
 
-// dK/dV workgroup: 4 waves = 2 key blocks x 2 query groups, each wave taking two
-// 32-row query blocks of a tile in turn.  With D = 64 two such workgroups share a
-// compute unit (two waves per SIMD); being independent they drift out of phase,
-// so one's matrix work overlaps the other's vector work and barrier waits.
+// dK/dV workgroup: 4 waves = 4 key blocks of 32 rows (kListBN keys); every wave takes the
+// four 32-row query blocks of a tile in turn, so a Q / dO tile fetched from L2 serves 128 keys
+// and nothing has to be summed across waves.  With D = 64 two such workgroups share a
+// compute unit (two waves per SIMD); being independent they drift out of phase, so one's
+// matrix work overlaps the other's vector work and barrier waits.
 template <int D> struct DkvShape {
-  static constexpr int kWaves = 4;
+  static constexpr int kWaves = kListBN / 32;
   static constexpr int kThreads = kWaves * 64;
-  static constexpr int kNQG = kWaves / 2;        // query groups
-  static constexpr int kQBlocks = 4 / kNQG;      // 32-row query blocks per wave and tile
+  static constexpr int kQBlocks = kBM / 32;        // 32-row query blocks per wave and tile
   static constexpr int kStages = D == 64 ? 2 : 1;  // LDS stages of the query-side tiles
 };
 
@@ -245,8 +250,8 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
                                                                T* __restrict__ dv) {
   typedef typename Frag<T>::vec8 vec8;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int BM = kBM, BN = kBN;
-  constexpr int kDkvThreads = DkvShape<D>::kThreads, NQG = DkvShape<D>::kNQG, QBW = DkvShape<D>::kQBlocks;
+  constexpr int BM = kBM, BN = kListBN;
+  constexpr int kDkvThreads = DkvShape<D>::kThreads, QBW = DkvShape<D>::kQBlocks;
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
   // LDS stages of (Q tile, dO tile, lse, -delta).  D = 64 keeps two, so that one workgroup
   // barrier per tile suffices; with D = 128 a second stage would cost the second workgroup
@@ -257,7 +262,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
-  const int wk = w & 1, wq = w >> 1;  // key block (32 rows) and query group of this wave
+  const int wk = w;  // key block (32 rows) of this wave
   const int nkt = (p.Lkv + BN - 1) / BN;
   int kt, bh;  // early key tiles see the most queries under causal masks
   xcd_tile_map(blockIdx.x, nkt, p.Hkv * p.B, kt, bh);
@@ -381,7 +386,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 #pragma unroll
       for (int qs = 0; qs < QBW; qs++) {
       // ---- S = Q.K^T and dP = dO.V^T for 32 query rows x 32 keys ----
-      const int qrow_w = (wq * QBW + qs) * 32;
+      const int qrow_w = qs * 32;
       float16_t sacc, dpacc;
       const int ql = qrow_w + 4 * g;  // local row of register 0
 #pragma unroll
@@ -453,37 +458,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
     }
   }
 
-  // sum the query groups of each key block through LDS: (3,2 -> 1,0 then) 1 -> 0
-  float* red = reinterpret_cast<float*>(bwd_smem);  // [2 slots][2 key blocks][2*DB*16 regs][64 lanes]
-  constexpr int kRegs = 2 * DB * 16;
-#pragma unroll
-  for (int round = (NQG == 4 ? 0 : 1); round < 2; round++) {
-    __syncthreads();
-    const bool writer = round == 0 ? (wq >= 2) : (wq == 1);
-    const bool reader = round == 0 ? (wq < 2) : (wq == 0);
-    const int slot = round == 0 ? (wq & 1) : 0;
-    float* base = red + ((size_t)(slot * 2 + wk) * kRegs) * 64 + lane;
-    if (writer) {
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          base[(db * 16 + r) * 64] = dkacc[db][r];
-          base[((DB + db) * 16 + r) * 64] = dvacc[db][r];
-        }
-    }
-    __syncthreads();
-    if (reader) {
-#pragma unroll
-      for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          dkacc[db][r] += base[(db * 16 + r) * 64];
-          dvacc[db][r] += base[((DB + db) * 16 + r) * 64];
-        }
-    }
-  }
-  if (wq == 0 && kv_col < p.Lkv) {
+  if (kv_col < p.Lkv) {
     const int64_t row_id = ((int64_t)b * p.Hkv + hk) * p.Lkv + kv_col;
     T* dkp = dk + row_id * D + 4 * g;
     T* dvp = dv + row_id * D + 4 * g;
@@ -505,15 +480,13 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 }
 
 template <int D, typename T> constexpr size_t dkv_smem() {
-  size_t tiles = DkvShape<D>::kStages * ((size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
-  size_t red = (size_t)2 * 2 * 2 * (D / 32) * 16 * 64 * sizeof(float);
-  return tiles > red ? tiles : red;
+  return DkvShape<D>::kStages * ((size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
 }
 
 template <typename T, int D, int KIND, bool RS>
 static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  const int nqt = (p.Lq + kBM - 1) / kBM, nkt = (p.Lkv + kBN - 1) / kBN;
+  const int nqt = (p.Lq + kBM - 1) / kBM, nkt = (p.Lkv + kListBN - 1) / kListBN;
   if (!(p.flags & FLEX_BWD_ONLY_DKV))
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
                        (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
@@ -575,7 +548,7 @@ bool flex_mfma_bwd_supported(const FlexAttnParams& p) {
   if (!flex_mfma_shape_ok(p)) return false;
   // the dK/dV kernel needs the transposed lists whenever lists are given
   const FlexTileLists& t = p.tiles_bwd;
-  if (t.kv_num && (t.q_block != kBM || t.kv_block != kBN)) return false;
+  if (t.kv_num && (t.q_block != kBM || t.kv_block != kListBN)) return false;
   if (t.kv_num && (!t.q_num || !t.q_idx || !t.full_q_num || !t.full_q_idx)) return false;
   return true;
 }

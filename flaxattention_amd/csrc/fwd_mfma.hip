@@ -598,7 +598,7 @@ bool flex_mfma_shape_ok(const FlexAttnParams& p) {
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
   const bool ok = (dtype == FLEX_F16 || dtype == FLEX_BF16) && D == Dv && (D == 64 || D == 128);
   *qb = !ok ? 0 : (which == 0 ? fwd_bm(D) : 128);
-  *kvb = ok ? kFwdBN : 0;
+  *kvb = !ok ? 0 : (which == 0 ? kFwdBN : 128);
 }
 
 bool flex_mfma_fwd_supported(const FlexAttnParams& p) {

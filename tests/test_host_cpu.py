@@ -59,7 +59,7 @@ def test_workspace_and_tile_queries_without_gpu():
     L.flexattn_preferred_tiles(_lib.FLEX_BF16, 128, 128, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (128, 64)
     L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 1, ctypes.byref(qb), ctypes.byref(kvb))
-    assert (qb.value, kvb.value) == (128, 64)
+    assert (qb.value, kvb.value) == (128, 128)
     L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (0, 0)
     # argument validation happens before anything touches a device
