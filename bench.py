@@ -76,7 +76,7 @@ class Prepared:
         if decode_splits:
             n = self.L.flexattn_decode_workspace_bytes(self.p, decode_splits)
             self.dws = torch.empty(max(n, 256), dtype=torch.uint8, device=dev)
-        self.stream = torch.cuda.current_stream(dev).cuda_stream
+        self.dev = dev
         self.ptr = {n: getattr(self, n).data_ptr() for n in ("q", "k", "v", "o", "lse", "d_o", "dq", "dk", "dv", "ws")}
         self.p_dq = self._with_flags(_lib.FLAG_BWD_ONLY_DQ)
         self.p_dkv = self._with_flags(_lib.FLAG_BWD_ONLY_DKV)
@@ -86,6 +86,11 @@ class Prepared:
         C.memmove(C.byref(p2), C.byref(self.p), C.sizeof(self.p))
         p2.flags = self.p.flags | extra
         return p2
+
+    @property
+    def stream(self):
+        # torch's current stream at call time, so that a capturing stream sees the launches
+        return torch.cuda.current_stream(self.dev).cuda_stream
 
     def fwd(self):
         t = self.ptr
@@ -179,7 +184,7 @@ def make_train_config(dev, name, opts=None):
     return pr, tiles, dtype
 
 
-def run_train_config(dev, name, steps, warmup, opts=None):
+def run_train_config(dev, name, steps, warmup, opts=None, graph=False):
     pr, tiles, dtype = make_train_config(dev, name, opts)
     per_tile = 128 * 128 * 64
     f_fwd, f_bwd = 4 * per_tile * tiles, 10 * per_tile * tiles
@@ -187,7 +192,19 @@ def run_train_config(dev, name, steps, warmup, opts=None):
     def step():
         pr.fwd()
         pr.bwd()
-    ms = wall_time_ms(step, steps, warmup)
+    if graph:
+        # the step is three kernel launches; replayed as one HIP graph (nothing in it allocates, synchronises
+        # or clears memory).  Measured no faster than eager launches here, so it is not the default.
+        step()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream(dev)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            step()
+        torch.cuda.synchronize()
+        ms = wall_time_ms(g.replay, steps, warmup)
+    else:
+        ms = wall_time_ms(step, steps, warmup)
     n = max(steps, 10)
     us = {"fwd_pipe_kernel": event_time_us(pr.fwd, n),
           "bwd_dq_kernel": event_time_us(lambda: pr.bwd("dq"), n),
@@ -215,6 +232,23 @@ def pmc_probe(dev, name, opts):
         pr.bwd("dq")
         pr.bwd("dkv")
     torch.cuda.synchronize()
+
+
+def run_mfma_probe(dev):
+    """Matrix throughput this GPU sustains on a kernel that only issues fp16 MFMAs on pseudo-random operands
+    (the library's measurement aid): the practical ceiling next to the published peak."""
+    from flaxattention_amd import _lib
+    L = _lib.lib()
+    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    flops = C.c_double(0.0)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def go():
+        rc = L.flexattn_probe_mfma(sink.data_ptr(), 4096, C.byref(flops), stream)
+        if rc:
+            _lib.check(rc, "flexattn_probe_mfma")
+    us = event_time_us(go, 20)
+    return flops.value / us / 1e6
 
 
 def run_config4(dev, steps, warmup):
@@ -259,6 +293,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--all", action="store_true", help="also run configurations 3, 4 and 5 (reported on stderr and in 'extra')")
     ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
+    ap.add_argument("--graph", action="store_true", help="replay the three kernels of a step as one HIP graph instead of launching them eagerly")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter run: one 1 GiB device copy (calibration) and 3 launches of each kernel of the workload, nothing else")
     a = ap.parse_args()
@@ -274,15 +309,18 @@ def main():
     if a.pmc_probe:
         pmc_probe(dev, a.workload, opts)
         return
-    r = run_train_config(dev, a.workload, a.steps, a.warmup, opts)
+    r = run_train_config(dev, a.workload, a.steps, a.warmup, opts, graph=a.graph)
     log(f"{a.workload}: {r['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r['tflops']:.1f} TFLOP/s  "
         f"(fwd {r['fwd_tflops']:.1f}, bwd {r['bwd_tflops']:.1f})  kernels {r['kernels']}")
     extra = {}
     if a.all:
         other = "config3" if a.workload == "config2" else "config2"
-        r2 = run_train_config(dev, other, a.steps, a.warmup, opts)
+        r2 = run_train_config(dev, other, a.steps, a.warmup, opts, graph=a.graph)
         log(f"{other}: {r2['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r2['tflops']:.1f} TFLOP/s  kernels {r2['kernels']}")
         extra[other] = {"ms_per_step": round(r2["ms_per_step"], 4), "fwd_bwd_tflops": round(r2["tflops"], 1), "kernels": r2["kernels"]}
+        probe = run_mfma_probe(dev)
+        log(f"MFMA-only probe kernel (fp16, pseudo-random operands): {probe:.0f} TFLOP/s sustained")
+        extra["mfma_probe_tflops"] = round(probe, 1)
         c4 = run_config4(dev, a.steps, a.warmup)
         log(f"config4: fwd {c4['us']:.1f} us  {c4['tflops']:.1f} TFLOP/s on {c4['tiles_per_head']} tiles/head")
         extra["config4"] = {"fwd_us": round(c4["us"], 1), "fwd_tflops": round(c4["tflops"], 1)}
@@ -302,7 +340,7 @@ def main():
         "dtype": r["dtype"], "data": "synthetic",
         "config": {"workload": {"config2": "configs[1]: fp16 [8,8,2048,64] checkerboard score_mod, no mask, forward + backward of out.sum()",
                                 "config3": "configs[2]: bf16 [8,8,2048,64] ALiBi score_mod, causal block mask 128x128, forward + backward of out.sum()"}[a.workload],
-                   "round_s": bool(a.round_s)},
+                   "round_s": bool(a.round_s), "launch": "hip graph replay" if a.graph else "eager"},
         "pct_mfma_peak": round(r["tflops"] / PEAK_MFMA_TFLOPS * 100, 2),
         "fwd_tflops": round(r["fwd_tflops"], 1), "bwd_tflops": round(r["bwd_tflops"], 1),
         "kernels": r["kernels"],

@@ -420,8 +420,13 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 #pragma unroll
   for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
 
+  const int slot = blockIdx.x >= (gridDim.x >> 1) ? 1 : 0;  // second half of the grid = second workgroup of a compute unit
   int st = 0;  // LDS stage of the current tile (it % 3)
   for (int it = 0; it < nt; it++) {
+    // Two workgroups share a compute unit and the instruction arbiter favours the older wave,
+    // which leaves the younger one behind until it runs alone at the end.  Trading the wave
+    // priority between them every tile keeps both advancing at the same pace.
+    if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
     const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
     const int st_n = st == 2 ? 0 : st + 1;
@@ -521,6 +526,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
     }
     st = st_n;
   }
+  __builtin_amdgcn_s_setprio(0);
   // the last unit's P is still pending
 #pragma unroll
   for (int tt = 0; tt < 2; tt++)

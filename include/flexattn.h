@@ -168,6 +168,13 @@ int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const
                     void* o, float* lse2, int32_t num_splits, void* workspace,
                     flexattn_stream_t stream);
 
+/* Measurement aid with no counterpart in the reference: launches a kernel that only
+ * issues v_mfma_f32_32x32x16_f16 on pseudo-random operands (512 workgroups x 4 waves,
+ * 8*iters MFMAs per wave) so that a caller can time the matrix throughput the GPU
+ * sustains under its power limit.  `sink` is a device buffer of 512*256 floats;
+ * *flops_per_launch receives the flop count of one launch. */
+int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, flexattn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
