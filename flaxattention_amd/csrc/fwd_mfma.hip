@@ -421,12 +421,17 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
 
   const int slot = blockIdx.x >= (gridDim.x >> 1) ? 1 : 0;  // second half of the grid = second workgroup of a compute unit
+  const bool trade = tl.kv_num == nullptr;
   int st = 0;  // LDS stage of the current tile (it % 3)
   for (int it = 0; it < nt; it++) {
     // Two workgroups share a compute unit and the instruction arbiter favours the older wave,
-    // which leaves the younger one behind until it runs alone at the end.  Trading the wave
-    // priority between them every tile keeps both advancing at the same pace.
-    if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
+    // which leaves the younger one behind until it runs alone at the end.  When all workgroups
+    // have the same amount of work (no tile lists), trading the wave priority between them
+    // every tile keeps both advancing at the same pace.  With lists the heavy workgroups are
+    // dispatched first and are the critical path, so the arbiter's preference is kept.
+    if (trade) {
+      if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
+    }
     const int kv0 = t_cur * BN;
     const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
     const int st_n = st == 2 ? 0 : st + 1;
