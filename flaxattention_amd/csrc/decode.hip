@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     kv_cur = kv_nx1;
     kv_nx1 = kv_nx2;
     if (st + 12 < st_end) kv_nx2 = step_kv0(st + 12);
-    const bool need_mask = !trivial_mask || (kv0 + kStep > p.Lkv);
+    // steps that come from the list of fully visible tiles need no mask evaluation
+    const bool listed_full = full_idx && (st >> 1) < n_full;
+    const bool need_mask = (!trivial_mask && !listed_full) || (kv0 + kStep > p.Lkv);
 
     vec8 pf[NB][2];
 #pragma unroll
@@ -164,8 +166,12 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
         sacc[r + 1] = sm[nb].apply_sub(s1, acc_row(r + 1), m_use);
       }
       if (need_mask) {
+        // a real branch whose inputs pass through the asm, so that none of the mask
+        // arithmetic can be hoisted into the unmasked path
+        int q_opaque = col_q[nb], kv_opaque = kv0;
+        asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
         Mask2 visible(p.mask, b, col_h[nb], p.Lkv);
-        mask_block_q(sacc, p.mask, visible, col_q[nb], kv0, g, p.Lkv);
+        mask_block_q(sacc, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
       }
       // online softmax; the reference max moves only when it is beaten by 2^kTau
       const float m_rel = xhalf_max(block_max(sacc));
@@ -365,10 +371,12 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 }
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
-  // aim for three workgroups per CU (256 CUs; the kernel fits three waves per SIMD), at least 8 steps each
+  // aim for one resident generation of workgroups on 256 CUs: three per CU with up to 32 query
+  // columns (three waves per SIMD), two per CU with 64; at least 8 steps each
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
-  int s = (int)((768 + heads - 1) / heads);
+  const int slots = (p.Hq / p.Hkv) * p.Lq > 32 ? 512 : 768;
+  int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
   if (s > 64) s = 64;
