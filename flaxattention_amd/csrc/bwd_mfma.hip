@@ -4,8 +4,8 @@
 // (flaxattention/kernel/attention.py:338-553) and of jax.grad through the dense
 // path.  P is recomputed from the saved base-2 log-sum-exp.  Two kernels:
 //
-//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 64
-//                  (two per entry of the 128-granular backward lists).  Transposed products keep one query
+//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 128
+//                  (the entries of the 128-granular backward lists).  Transposed products keep one query
 //                  row per lane, so lse and delta are per-lane scalars:
 //                    S^T = K.Q^T,  dP^T = V.dO^T,  dS^T = P^T o (dP^T - delta) * g,
 //                    dQ^T += K^T.dS^T.
@@ -20,7 +20,7 @@
 namespace flex {
 
 constexpr int kBM = 128;     // query tile (list granularity)
-constexpr int kBN = 64;      // key tile staged per step by the dQ kernel
+constexpr int kBN = 128;     // key tile staged per step by the dQ kernel
 constexpr int kListBN = 128; // key granularity of the backward tile lists = key rows of a dK/dV workgroup
 
 template <typename T, int D, int KIND, bool ROUND_S>
@@ -152,7 +152,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
     // one 32-key block at a time (S, dP, softmax, dQ): half the accumulator registers of
     // doing both blocks side by side
 #pragma unroll
-    for (int nb = 0; nb < 2; nb++) {
+    for (int nb = 0; nb < BN / 32; nb++) {
       // dP starts at -delta, so the accumulator comes out as dP - delta
       float16_t sacc, dpacc, gacc;
 #pragma unroll
