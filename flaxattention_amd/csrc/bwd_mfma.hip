@@ -487,9 +487,17 @@ template <typename T, int D, int KIND, bool RS>
 static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
   const int nqt = (p.Lq + kBM - 1) / kBM, nkt = (p.Lkv + kListBN - 1) / kListBN;
-  if (!(p.flags & FLEX_BWD_ONLY_DKV))
-    hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
-                       (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+  if (!(p.flags & FLEX_BWD_ONLY_DKV)) {
+    if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.p0 > 0.f && p.score.p1 > 0.f) {
+      // positive factors: the derivative folds into the exponent
+      constexpr int KF = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardFold : KIND;
+      hipLaunchKernelGGL((bwd_dq_kernel<T, D, KF, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
+                         (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+    } else {
+      hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
+                         (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+    }
+  }
   if (p.flags & FLEX_BWD_ONLY_DQ) return 0;
   constexpr size_t sm = dkv_smem<D, T>();
   static bool attr_set = false;

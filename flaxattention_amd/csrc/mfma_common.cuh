@@ -126,6 +126,29 @@ template <> struct Score2<kScoreCheckerboardKv> {
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
+// Checkerboard with positive factors, for a kernel that only needs dS = P o (dP - delta) o g
+// (dQ): the derivative g is the factor itself, and P.g = 2^(x + log2 g), so log2 g joins the
+// constant subtracted in the exponent and the derivative costs nothing per element.
+constexpr int kScoreCheckerboardFold = 101;
+template <> struct Score2<kScoreCheckerboardFold> {
+  static constexpr bool kGradOne = true;  // folded into the exponent
+  float c0, c1, l0, l1;
+  float ce, co, le, lo;
+  int by_kv;
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+    c0 = m.p0 * scale * kLog2e; c1 = m.p1 * scale * kLog2e; l0 = log2f(m.p0); l1 = log2f(m.p1); by_kv = m.i0;
+  }
+  __device__ __forceinline__ void tile(int q, int kvb) {
+    int par = (by_kv ? kvb : (kvb - q)) & 1;  // parity at off = 0
+    ce = par ? c1 : c0; co = par ? c0 : c1;
+    le = par ? l1 : l0; lo = par ? l0 : l1;
+  }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const {
+    return (off & 1) ? fmaf(s, co, lo - m) : fmaf(s, ce, le - m);
+  }
+  __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
+};
+
 template <> struct Score2<FLEX_SCORE_ALIBI> {
   static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;

@@ -66,3 +66,18 @@ def test_decode_matches_prefill_kernel(dev):
     a = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(8, -1.0), block_mask=bm, kernel_options={"decode_splits": 16})
     b = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(8, -1.0), block_mask=bm, kernel_options={"decode_splits": 0, "decode": False})
     assert max_abs(a.cpu(), b.cpu()) <= 4e-3
+
+
+def test_mfma_probe_runs(dev):
+    """The measurement aid launches, reports its flop count and leaves finite values behind."""
+    import ctypes
+    from flaxattention_amd import _lib
+    L = _lib.lib()
+    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    flops = ctypes.c_double(0.0)
+    rc = L.flexattn_probe_mfma(sink.data_ptr(), 4, ctypes.byref(flops), torch.cuda.current_stream(dev).cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert flops.value == 512 * 4 * 8 * 4 * 2 * 32 * 32 * 16
+    assert torch.isfinite(sink).all()
+    assert L.flexattn_probe_mfma(None, 4, None, None) != 0 and b"probe" in L.flexattn_last_error()
