@@ -17,6 +17,9 @@ selects numerics here:
                         (default True, as attention.py:27 computes that product
                         in the input dtype)
     {"backend": "generic" | "auto"}
+    {"decode": bool}      split-KV decode kernel on / off; by default it is used
+                          whenever it applies (fp16/bf16, D = Dv in {64, 128},
+                          at most 64 query rows per KV head, at least 512 keys)
     {"decode_splits": n}  force the split-KV decode kernel with n splits
 """
 from __future__ import annotations
@@ -85,6 +88,8 @@ class _Plan:
         self.Hkv, self.Lkv, self.Dv = k.shape[1], k.shape[2], v.shape[3]
         self.dtype = q.dtype
         self.score, self.mask, self.block_mask = score, mask, block_mask
+        # decode_splits: > 0 = decode kernel with that many splits, < 0 = decode kernel with the
+        # library's default split count, 0 = forward kernel
         self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
         self.lists = None       # tile lists for the forward / decode kernels
         self.lists_bwd = None   # tile lists for the backward kernels
@@ -135,8 +140,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
         flags |= _lib.FLAG_ROUND_S
     if opts.get("backend", "auto") == "generic":
         flags |= _lib.FLAG_FORCE_GENERIC
-    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True,
-                 opts.get("decode_splits", 0) if opts.get("decode", True) else 0)
+    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, flags, opts))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
         holder = block_mask if block_mask is not None else _holder_for(mask)
@@ -152,6 +156,21 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
                 else:
                     plan.lists_bwd = lists
     return plan
+
+
+def _decode_choice(q, k, v, flags: int, opts: dict) -> int:
+    """Split count for the decode kernel (> 0 given, < 0 library default) or 0 for the forward kernel."""
+    if int(opts.get("decode_splits", 0)) > 0:
+        return int(opts["decode_splits"])
+    want = opts.get("decode")
+    if want is False:
+        return 0
+    Hq, Lq, D = q.shape[1], q.shape[2], q.shape[3]
+    fits = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
+            and (Hq // k.shape[1]) * Lq <= 64 and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
+    if want is True:
+        return -1   # the library reports what does not fit
+    return -1 if fits and k.shape[2] >= 512 else 0
 
 
 _holders: dict = {}
@@ -182,11 +201,12 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     lse2 = torch.empty((plan.B, plan.Hq, plan.Lq), dtype=torch.float32, device=q.device)
     p = plan.params(q, k, v, o)
     with torch.cuda.device(q.device):
-        if plan.decode_splits > 0:
-            nbytes = L.flexattn_decode_workspace_bytes(p, plan.decode_splits)
+        if plan.decode_splits != 0:
+            splits = max(plan.decode_splits, 0)   # 0 asks the library for its default
+            nbytes = L.flexattn_decode_workspace_bytes(p, splits)
             ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
             rc = L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(),
-                                   plan.decode_splits, ws.data_ptr(), _stream(q))
+                                   splits, ws.data_ptr(), _stream(q))
             _lib.check(rc, "flexattn_decode")
         else:
             rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), None, _stream(q))

@@ -81,3 +81,20 @@ def test_mfma_probe_runs(dev):
     assert flops.value == 512 * 4 * 8 * 4 * 2 * 32 * 32 * 16
     assert torch.isfinite(sink).all()
     assert L.flexattn_probe_mfma(None, 4, None, None) != 0 and b"probe" in L.flexattn_last_error()
+
+
+def test_decode_is_chosen_automatically(dev):
+    """Short queries against a long KV cache take the decode kernel without being asked;
+    {"decode": False} keeps the forward kernel; both agree, and the gradient path is unaffected."""
+    from flaxattention_amd.core.attention import _make_plan
+    q, k, v = (t.to(dev) for t in seeded_qkv(2, 4, 4, 4, 1024, 64, torch.float16))
+    assert _make_plan(q, k, v, None, None, None, 0.125, None).decode_splits < 0
+    assert _make_plan(q, k, v, None, None, None, 0.125, {"decode": False}).decode_splits == 0
+    assert _make_plan(q, k[:, :, :256], v[:, :, :256], None, None, None, 0.125, None).decode_splits == 0
+    assert _make_plan(q.float(), k.float(), v.float(), None, None, None, 0.125, None).decode_splits == 0
+    qg = q.clone().requires_grad_(True)
+    a = fa.flax_attention(qg, k, v, score_mod=generate_alibi_bias(4))
+    b = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(4), kernel_options={"decode": False})
+    assert max_abs(a.detach().cpu(), b.cpu()) <= 2e-3
+    a.sum().backward()
+    assert torch.isfinite(qg.grad).all() and qg.grad.abs().max() > 0
