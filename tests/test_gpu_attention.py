@@ -276,3 +276,40 @@ def test_fused_decode_shapes_through_prefill_kernel(dev):
     for ql in (1, 16, 64):
         run(dev, torch.float16, 2, 4, 4, ql, 1024, 64, score=generate_alibi_bias(4, -1.0), oscore=o_alibi_config(4),
             mask=offset_causal_mask(1024 - ql), omask=o_offset_causal(1024 - ql), strict=False, grad=False)
+
+
+# ---- seeded sweep over shapes x functors for the fused kernels (forward, dQ, dK, dV, lse) ----
+def _sweep_case(seed):
+    import random
+    rnd = random.Random(1000 + seed)
+    dtype = rnd.choice([torch.float16, torch.float16, torch.bfloat16])
+    D = rnd.choice([64, 64, 128])
+    Hkv = rnd.choice([1, 2, 3])
+    G = rnd.choice([1, 1, 2, 4])
+    B = rnd.choice([1, 2])
+    Lq = rnd.choice([1, 17, 64, 129, 256, 300, 511, 640])
+    Lkv = rnd.choice([33, 64, 200, 257, 512, 600, 777])
+    name, score, oscore = rnd.choice([s for s in SCORES if s[0] != "alibi_ref"])
+    if name.startswith("alibi"):   # the slope table depends on the head count
+        score, oscore = (generate_alibi_bias(Hkv * G, sign=-1.0), o_alibi_config(Hkv * G))
+    w = rnd.choice([16, 40, 130])
+    masks = [(None, None), (causal_mask, o_causal_mask), (generate_sliding_window(w), o_sliding_window(w)),
+             (generate_attention_sink(w, 4), o_attention_sink(w, 4)),
+             (offset_causal_mask(max(Lkv - Lq, 0)), o_offset_causal(max(Lkv - Lq, 0)))]
+    mask, omask = rnd.choice(masks)
+    return dict(dtype=dtype, B=B, Hq=Hkv * G, Hkv=Hkv, Lq=Lq, Lkv=Lkv, D=D, score=score, oscore=oscore, mask=mask,
+                omask=omask, use_block_mask=rnd.random() < 0.7, pallas=False, name=name)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_fused_seeded_sweep(dev, seed):
+    c = _sweep_case(seed)
+    print(f"sweep {seed}: {c['dtype']} B{c['B']} Hq{c['Hq']} Hkv{c['Hkv']} Lq{c['Lq']} Lkv{c['Lkv']} D{c['D']} "
+          f"score {c['name']} mask {getattr(c['mask'], '__name__', c['mask'])} block_mask {c['use_block_mask']}", flush=True)
+    if c["mask"] is not None and not c["use_block_mask"]:
+        # a bare mask_mod goes through flax_attention_pallas (flax_attention takes block masks only)
+        run(dev, c["dtype"], c["B"], c["Hq"], c["Hkv"], c["Lq"], c["Lkv"], c["D"], score=c["score"], oscore=c["oscore"],
+            mask=c["mask"], omask=c["omask"], strict=False, pallas=True, scale_maxabs=True)
+    else:
+        run(dev, c["dtype"], c["B"], c["Hq"], c["Hkv"], c["Lq"], c["Lkv"], c["D"], score=c["score"], oscore=c["oscore"],
+            mask=c["mask"], omask=c["omask"], strict=False, scale_maxabs=True)
