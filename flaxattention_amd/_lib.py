@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("FLEXATTN_LIB") or os.path.join(_HERE, "libflexattn.so
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
 FLEX_F32, FLEX_F16, FLEX_BF16 = 0, 1, 2
-SCORE_IDENTITY, SCORE_CHECKERBOARD, SCORE_ALIBI, SCORE_TANH_SOFTCAP, SCORE_REL_BIAS = range(5)
+SCORE_IDENTITY, SCORE_CHECKERBOARD, SCORE_ALIBI, SCORE_TANH_SOFTCAP, SCORE_REL_BIAS, SCORE_AFFINE = range(6)
 MASK_BAND, MASK_BITS = 0, 1
 FLAG_ROUND_S, FLAG_STRICT, FLAG_FORCE_GENERIC, FLAG_BWD_ONLY_DQ, FLAG_BWD_ONLY_DKV = 1, 2, 4, 8, 16
 INT_MIN, INT_MAX = -(2 ** 31), 2 ** 31 - 1
@@ -23,7 +23,9 @@ INT_MIN, INT_MAX = -(2 ** 31), 2 ** 31 - 1
 
 class FlexScoreMod(C.Structure):
     _fields_ = [("kind", C.c_int32), ("p0", C.c_float), ("p1", C.c_float),
-                ("i0", C.c_int32), ("i1", C.c_int32)]
+                ("i0", C.c_int32), ("i1", C.c_int32),
+                ("mul", C.c_void_p), ("add", C.c_void_p),
+                ("stride_b", C.c_int64), ("stride_h", C.c_int64), ("stride_q", C.c_int64)]
 
 
 class FlexMask(C.Structure):

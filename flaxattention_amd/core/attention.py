@@ -93,7 +93,7 @@ class _Plan:
         self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
         self.lists = None       # tile lists for the forward / decode kernels
         self.lists_bwd = None   # tile lists for the backward kernels
-        self.keep = [mask.bits]
+        self.keep = [mask.bits, score.mul, score.add]
 
     def params(self, q, k, v, o) -> _lib.FlexAttnParams:
         p = _lib.FlexAttnParams()
@@ -125,7 +125,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
     B, Hq, Lq, D = q.shape
     Lkv = k.shape[2]
     dev = q.device
-    score = resolve_score_mod(score_mod, Hq)
+    score = resolve_score_mod(score_mod, Hq, (B, Hq, Lq, Lkv), dev)
     if block_mask is not None:
         if block_mask.seq_lengths is not None and (block_mask.seq_lengths[0] < Lq or block_mask.seq_lengths[1] < Lkv):
             raise ValueError(f"block_mask was built for lengths {block_mask.seq_lengths}, "
@@ -140,7 +140,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
         flags |= _lib.FLAG_ROUND_S
     if opts.get("backend", "auto") == "generic":
         flags |= _lib.FLAG_FORCE_GENERIC
-    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, flags, opts))
+    plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, score, flags, opts))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
         holder = block_mask if block_mask is not None else _holder_for(mask)
@@ -158,7 +158,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
     return plan
 
 
-def _decode_choice(q, k, v, flags: int, opts: dict) -> int:
+def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
     """Split count for the decode kernel (> 0 given, < 0 library default) or 0 for the forward kernel."""
     if int(opts.get("decode_splits", 0)) > 0:
         return int(opts["decode_splits"])
@@ -167,7 +167,8 @@ def _decode_choice(q, k, v, flags: int, opts: dict) -> int:
         return 0
     Hq, Lq, D = q.shape[1], q.shape[2], q.shape[3]
     fits = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
-            and (Hq // k.shape[1]) * Lq <= 64 and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
+            and (Hq // k.shape[1]) * Lq <= 64 and score.kind != _lib.SCORE_AFFINE
+            and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
     if want is True:
         return -1   # the library reports what does not fit
     return -1 if fits and k.shape[2] >= 512 else 0

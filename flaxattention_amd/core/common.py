@@ -15,7 +15,7 @@ from __future__ import annotations
 import inspect
 import math
 from enum import Enum
-from typing import Any, Callable, Optional
+from typing import Any, Callable, Optional, Tuple
 
 import torch
 
@@ -68,14 +68,26 @@ class ScoreMod:
     kind/p0/p1/i0 are the fields of FlexScoreMod.  Calling the object applies
     the same scalar function to its arguments."""
 
-    def __init__(self, kind: int, p0: float = 0.0, p1: float = 0.0, i0: int = 0, name: str = "score_mod"):
+    def __init__(self, kind: int, p0: float = 0.0, p1: float = 0.0, i0: int = 0, name: str = "score_mod",
+                 mul: Optional[torch.Tensor] = None, add: Optional[torch.Tensor] = None, fn: Optional[Callable] = None):
         self.kind, self.p0, self.p1, self.i0 = int(kind), float(p0), float(p1), int(i0)
         self.__name__ = name
+        # SCORE_AFFINE: dense fp32 tables [b', h', q', Lkv] (each leading extent 1 or full) and the
+        # callable they were read from
+        self.mul, self.add, self.fn = mul, add, fn
 
     def c_struct(self) -> _lib.FlexScoreMod:
-        return _lib.FlexScoreMod(self.kind, self.p0, self.p1, self.i0, 0)
+        m = _lib.FlexScoreMod(self.kind, self.p0, self.p1, self.i0, 0)
+        t = self.mul if self.mul is not None else self.add
+        if t is not None:
+            m.mul = self.mul.data_ptr() if self.mul is not None else None
+            m.add = self.add.data_ptr() if self.add is not None else None
+            m.stride_b, m.stride_h, m.stride_q = (t.stride(i) if t.shape[i] > 1 else 0 for i in range(3))
+        return m
 
     def key(self):
+        if self.kind == _lib.SCORE_AFFINE:
+            return (self.kind, id(self.mul), id(self.add))
         return (self.kind, self.p0, self.p1, self.i0)
 
     def __call__(self, score, b, h, q_idx, kv_idx):
@@ -96,6 +108,8 @@ class ScoreMod:
             return self.p0 * math.tanh(score / self.p0)
         if k == _lib.SCORE_REL_BIAS:
             return score + _f32(kv_idx - q_idx) * self.p0
+        if k == _lib.SCORE_AFFINE:
+            return self.fn(score, b, h, q_idx, kv_idx)
         raise ValueError(f"unknown score_mod kind {k}")
 
     def __repr__(self):
@@ -159,11 +173,58 @@ def _probe_score_mod(fn: Callable, H: int) -> Optional[ScoreMod]:
     return None
 
 
+def affine_score_mod(fn: Callable, B: int, H: int, Lq: int, Lkv: int, device) -> Optional[ScoreMod]:
+    """Lower a score_mod that is affine in the score, mod(s) = mul[b,h,q,kv] * s + add[b,h,q,kv], to dense
+    fp32 tables read off the callable on the device (what attention.py:59-63 evaluates per element;
+    captured tensors such as bias tables, attention.py:22-23, are simply part of the callable).
+    Returns None when the callable is not affine in the score."""
+    # affinity, on a small CPU grid: five score values must lie on one line per (b, h, q, kv)
+    P = 5
+    s = torch.tensor([-1.75, -0.5, 0.0, 0.625, 2.5], dtype=torch.float32).reshape(5, 1, 1, 1, 1)
+    b = torch.arange(min(B, 2), dtype=torch.int32).reshape(1, -1, 1, 1, 1)
+    h = torch.arange(H, dtype=torch.int32).reshape(1, 1, H, 1, 1)
+    q = torch.arange(min(Lq, P), dtype=torch.int32).reshape(1, 1, 1, -1, 1)
+    kv = torch.arange(min(Lkv, P + 2), dtype=torch.int32).reshape(1, 1, 1, 1, -1)
+    shape = (5, b.numel(), H, q.numel(), kv.numel())
+    try:
+        out = torch.broadcast_to(torch.as_tensor(fn(s.expand(shape), b, h, q, kv)).to(torch.float32), shape)
+    except Exception:
+        return None
+    a0, c0 = (out[4] - out[2]) / 2.5, out[2]
+    if not torch.isfinite(out).all() or not torch.allclose(out, a0 * s + c0, rtol=1e-5, atol=1e-5):
+        return None
+    # the tables, on the device; a [1,1,1,1] score keeps every extent the callable does not use at 1
+    bi = torch.arange(B, dtype=torch.int32, device=device).reshape(B, 1, 1, 1)
+    hi = torch.arange(H, dtype=torch.int32, device=device).reshape(1, H, 1, 1)
+    qi = torch.arange(Lq, dtype=torch.int32, device=device).reshape(1, 1, Lq, 1)
+    ki = torch.arange(Lkv, dtype=torch.int32, device=device).reshape(1, 1, 1, Lkv)
+    zero = torch.zeros((1, 1, 1, 1), dtype=torch.float32, device=device)
+    add = torch.as_tensor(fn(zero, bi, hi, qi, ki)).to(torch.float32)
+    # slope from a wide symmetric difference: the additive part cancels with little rounding left
+    mul = (torch.as_tensor(fn(zero + 8.0, bi, hi, qi, ki)).to(torch.float32)
+           - torch.as_tensor(fn(zero - 8.0, bi, hi, qi, ki)).to(torch.float32)) / 16.0
+    while add.dim() < 4:
+        add = add.unsqueeze(0)
+    while mul.dim() < 4:
+        mul = mul.unsqueeze(0)
+    full = (B, H, Lq, Lkv)
+    shp = tuple(max(add.shape[i], mul.shape[i]) for i in range(3)) + (Lkv,)
+    if any(shp[i] not in (1, full[i]) for i in range(3)):
+        return None
+    add = None if not bool(add.any()) else torch.broadcast_to(add, shp).contiguous()
+    mul = None if bool(((mul - 1).abs() <= 1e-6).all()) else torch.broadcast_to(mul, shp).contiguous()
+    if add is None and mul is None:
+        return IDENTITY
+    return ScoreMod(_lib.SCORE_AFFINE, name=getattr(fn, "__name__", "affine_score_mod"), mul=mul, add=add, fn=fn)
+
+
 _score_cache: dict = {}
 
 
-def resolve_score_mod(fn: Optional[Callable], H: int) -> ScoreMod:
-    """Lower a score_mod callable to a kernel functor, or raise."""
+def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int, int, int, int]] = None,
+                      device=None) -> ScoreMod:
+    """Lower a score_mod callable to a kernel functor, or raise.  `shape` = (B, H, Lq, Lkv) and `device`
+    allow the dense affine form for callables outside the functor families."""
     if fn is None or fn is _identity:
         return IDENTITY
     if isinstance(fn, ScoreMod):
@@ -173,13 +234,24 @@ def resolve_score_mod(fn: Optional[Callable], H: int) -> ScoreMod:
     if hit is not None and hit[0] is fn:
         return hit[1]
     spec = _probe_score_mod(fn, H)
-    if spec is None:
-        raise NotImplementedError(
-            "score_mod is not one of the fused functor families (identity, checkerboard, ALiBi, "
-            "tanh soft-cap, relative-position bias); build it with flaxattention_amd.mods.* "
-            "so the kernels can fuse it")
-    _score_cache[key] = (fn, spec)
-    return spec
+    if spec is not None:
+        _score_cache[key] = (fn, spec)
+        return spec
+    if shape is not None and device is not None:
+        key = (id(fn),) + tuple(shape) + (str(device),)
+        hit = _score_cache.get(key)
+        if hit is not None and hit[0] is fn:
+            return hit[1]
+        spec = affine_score_mod(fn, *shape, device)
+        if spec is not None:
+            if len(_score_cache) > 64:
+                _score_cache.clear()
+            _score_cache[key] = (fn, spec)
+            return spec
+    raise NotImplementedError(
+        "score_mod is neither one of the fused functor families (identity, checkerboard, ALiBi, tanh soft-cap, "
+        "relative-position bias) nor affine in the score (mul[b,h,q,kv] * score + add[b,h,q,kv]); "
+        "only those can be lowered to the kernels")
 
 
 # ---------------------------------------------------------------------------

@@ -38,12 +38,24 @@ struct ScoreArgs {
   float p0, p1;
   int32_t i0;
   float slope;  // ALiBi: exp2(-(h+1)*8/H) of the current head
+  const float* mul_bh;  // affine tables of the current (b, h), or null
+  const float* add_bh;
+  int64_t stride_q;
+  int32_t q_last, kv_last;  // table bounds: kernels evaluate functors on padded indices too
 };
 
-__device__ __forceinline__ ScoreArgs make_score_args(const FlexScoreMod& m, int h) {
+__device__ __forceinline__ ScoreArgs make_score_args(const FlexScoreMod& m, int b, int h, int Lq, int Lkv) {
   ScoreArgs a;
   a.p0 = m.p0; a.p1 = m.p1; a.i0 = m.i0; a.slope = 0.f;
+  a.mul_bh = nullptr; a.add_bh = nullptr; a.stride_q = 0;
+  a.q_last = Lq - 1; a.kv_last = Lkv - 1;
   if (m.kind == FLEX_SCORE_ALIBI) a.slope = exp2f(-((float)(h + 1) * 8.0f / (float)m.i0));
+  if (m.kind == FLEX_SCORE_AFFINE) {
+    const int64_t off = b * m.stride_b + h * m.stride_h;
+    a.mul_bh = m.mul ? m.mul + off : nullptr;
+    a.add_bh = m.add ? m.add + off : nullptr;
+    a.stride_q = m.stride_q;
+  }
   return a;
 }
 
@@ -89,6 +101,21 @@ template <> struct ScoreMod<FLEX_SCORE_REL_BIAS> {
   static __device__ __forceinline__ float grad(float s, int q, int kv, const ScoreArgs&) { return 1.f; }
 };
 
+template <> struct ScoreMod<FLEX_SCORE_AFFINE> {
+  // indices past the end (padding rows / columns of a chunk, masked out by the caller) are clamped
+  static __device__ __forceinline__ int64_t at(int q, int kv, const ScoreArgs& a) {
+    return (int64_t)min(max(q, 0), a.q_last) * a.stride_q + min(max(kv, 0), a.kv_last);
+  }
+  static __device__ __forceinline__ float mul(int q, int kv, const ScoreArgs& a) {
+    return a.mul_bh ? a.mul_bh[at(q, kv, a)] : 1.f;
+  }
+  static __device__ __forceinline__ float apply(float s, int q, int kv, const ScoreArgs& a) {
+    const float c = a.add_bh ? a.add_bh[at(q, kv, a)] : 0.f;
+    return fmaf(s, mul(q, kv, a), c);
+  }
+  static __device__ __forceinline__ float grad(float s, int q, int kv, const ScoreArgs& a) { return mul(q, kv, a); }
+};
+
 // runtime dispatch for the kernels that are not templated on the functor
 __device__ __forceinline__ float score_apply(int kind, float s, int q, int kv, const ScoreArgs& a) {
   switch (kind) {
@@ -96,6 +123,7 @@ __device__ __forceinline__ float score_apply(int kind, float s, int q, int kv, c
     case FLEX_SCORE_ALIBI: return ScoreMod<FLEX_SCORE_ALIBI>::apply(s, q, kv, a);
     case FLEX_SCORE_TANH_SOFTCAP: return ScoreMod<FLEX_SCORE_TANH_SOFTCAP>::apply(s, q, kv, a);
     case FLEX_SCORE_REL_BIAS: return ScoreMod<FLEX_SCORE_REL_BIAS>::apply(s, q, kv, a);
+    case FLEX_SCORE_AFFINE: return ScoreMod<FLEX_SCORE_AFFINE>::apply(s, q, kv, a);
     default: return s;
   }
 }
@@ -103,6 +131,7 @@ __device__ __forceinline__ float score_grad(int kind, float s, int q, int kv, co
   switch (kind) {
     case FLEX_SCORE_CHECKERBOARD: return ScoreMod<FLEX_SCORE_CHECKERBOARD>::grad(s, q, kv, a);
     case FLEX_SCORE_TANH_SOFTCAP: return ScoreMod<FLEX_SCORE_TANH_SOFTCAP>::grad(s, q, kv, a);
+    case FLEX_SCORE_AFFINE: return ScoreMod<FLEX_SCORE_AFFINE>::grad(s, q, kv, a);
     default: return 1.f;
   }
 }

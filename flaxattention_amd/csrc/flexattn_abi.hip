@@ -39,9 +39,10 @@ static int validate(const FlexAttnParams* p, const char* who) {
   }
   if (p->Hq % p->Hkv != 0) { flex_set_error("%s: Hq=%d is not a multiple of Hkv=%d", who, p->Hq, p->Hkv); return 1; }
   if (p->Dv > p->D) { flex_set_error("%s: Dv=%d must be <= D=%d", who, p->Dv, p->D); return 1; }
-  if (p->score.kind < FLEX_SCORE_IDENTITY || p->score.kind > FLEX_SCORE_REL_BIAS) { flex_set_error("%s: unknown score_mod kind %d", who, p->score.kind); return 1; }
+  if (p->score.kind < FLEX_SCORE_IDENTITY || p->score.kind > FLEX_SCORE_AFFINE) { flex_set_error("%s: unknown score_mod kind %d", who, p->score.kind); return 1; }
   if (p->score.kind == FLEX_SCORE_ALIBI && p->score.i0 <= 0) { flex_set_error("%s: ALiBi needs the head count in i0", who); return 1; }
   if (p->score.kind == FLEX_SCORE_TANH_SOFTCAP && !(p->score.p0 > 0.f)) { flex_set_error("%s: tanh soft-cap needs cap > 0", who); return 1; }
+  if (p->score.kind == FLEX_SCORE_AFFINE && !p->score.mul && !p->score.add) { flex_set_error("%s: affine score_mod without tables", who); return 1; }
   if (p->mask.kind != FLEX_MASK_BAND && p->mask.kind != FLEX_MASK_BITS) { flex_set_error("%s: unknown mask kind %d", who, p->mask.kind); return 1; }
   if (p->mask.kind == FLEX_MASK_BITS && !p->mask.bits) { flex_set_error("%s: bitmap mask without bits", who); return 1; }
   const FlexTileLists* both[2] = {&p->tiles, &p->tiles_bwd};

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(kWaves * 64) void generic_fwd_kernel(FlexAttnParams
   if (row_ok) for (int x = lane; x < D; x += 64) qf[x] = (float)qrow[x];
 
   RowCtx c;
-  c.kind = p.score.kind; c.sa = make_score_args(p.score, h); c.scale = p.scale;
+  c.kind = p.score.kind; c.sa = make_score_args(p.score, b, h, p.Lq, p.Lkv); c.scale = p.scale;
   c.round_s = (p.flags & (FLEX_ROUND_S | FLEX_STRICT)) != 0;
   const bool strict = (p.flags & FLEX_STRICT) != 0;
   MaskEval visible(p.mask, b, h);
@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kWaves * 64) void generic_dq_kernel(FlexAttnParams 
     for (int x = lane; x < Dv; x += 64) dof[x] = (float)dorow[x];
   }
   RowCtx c;
-  c.kind = p.score.kind; c.sa = make_score_args(p.score, h); c.scale = p.scale;
+  c.kind = p.score.kind; c.sa = make_score_args(p.score, b, h, p.Lq, p.Lkv); c.scale = p.scale;
   c.round_s = (p.flags & (FLEX_ROUND_S | FLEX_STRICT)) != 0;
   const bool strict = (p.flags & FLEX_STRICT) != 0;
   MaskEval visible(p.mask, b, h);
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(kWaves * 64) void generic_dkv_kernel(FlexAttnParams
   for (int g = 0; g < G; g++) {
     const int h = hk * G + g;
     RowCtx c;
-    c.kind = p.score.kind; c.sa = make_score_args(p.score, h); c.scale = p.scale;
+    c.kind = p.score.kind; c.sa = make_score_args(p.score, b, h, p.Lq, p.Lkv); c.scale = p.scale;
     c.round_s = (p.flags & (FLEX_ROUND_S | FLEX_STRICT)) != 0;
     MaskEval visible(p.mask, b, h);
     const T* qbase = q + b * p.q_stride[0] + h * p.q_stride[1];

@@ -35,13 +35,23 @@ enum FlexScoreKind {
   FLEX_SCORE_ALIBI = 2,        /* flaxattention/mods/alibi.py:15-18:
                                   score + p0*(q_idx-kv_idx)*exp2(-(h+1)*8/i0) */
   FLEX_SCORE_TANH_SOFTCAP = 3, /* p0 * tanh(score / p0) */
-  FLEX_SCORE_REL_BIAS = 4      /* score + p0 * (kv_idx - q_idx) */
+  FLEX_SCORE_REL_BIAS = 4,     /* score + p0 * (kv_idx - q_idx) */
+  FLEX_SCORE_AFFINE = 5        /* mul[b,h,q,kv] * score + add[b,h,q,kv] from dense fp32
+                                  tables: what a Python score_mod that is affine in the score
+                                  (captured bias tables, position-dependent scaling;
+                                  attention.py:22-23, 59-63) is lowered to.  Served by the
+                                  generic kernels only. */
 };
 
 typedef struct FlexScoreMod {
   int32_t kind;
   float p0, p1;
   int32_t i0, i1;
+  /* FLEX_SCORE_AFFINE: tables indexed [b*stride_b + h*stride_h + q*stride_q + kv]
+   * (strides in elements, 0 broadcasts); a NULL mul means 1, a NULL add means 0 */
+  const float* mul;
+  const float* add;
+  int64_t stride_b, stride_h, stride_q;
 } FlexScoreMod;
 
 /* mask_mod functors (flaxattention/core/common.py:8).  FLEX_MASK_BAND is a

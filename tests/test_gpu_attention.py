@@ -313,3 +313,28 @@ def test_fused_seeded_sweep(dev, seed):
     else:
         run(dev, c["dtype"], c["B"], c["Hq"], c["Hkv"], c["Lq"], c["Lkv"], c["D"], score=c["score"], oscore=c["oscore"],
             mask=c["mask"], omask=c["omask"], strict=False, scale_maxabs=True)
+
+
+# ---- score_mods outside the functor families: lowered to dense affine tables, generic kernels ----
+def test_affine_score_mod_tables(dev):
+    table = torch.randn(4, 31, generator=torch.Generator().manual_seed(7))
+    table_dev = table.to(dev)
+
+    def rel_table(score, b, h, q_idx, kv_idx):   # learned relative-position bias (a captured buffer)
+        t = table_dev if score.is_cuda else table
+        return score + t[h.long(), (q_idx - kv_idx).clamp(-15, 15).long() + 15]
+
+    def block_scale(score, b, h, q_idx, kv_idx):  # position-dependent scaling plus a per-batch shift
+        return torch.where(q_idx // 32 == kv_idx // 32, score, score * 0.5) + 0.25 * b
+
+    for fn in (rel_table, block_scale):
+        for dtype in (torch.float32, torch.float16):
+            print(f"case affine {fn.__name__} {dtype}", flush=True)
+            run(dev, dtype, 2, 4, 2, 70, 150, 64, score=fn, oscore=fn, mask=causal_mask, omask=o_causal_mask,
+                strict=(dtype == torch.float16), opts=None if dtype == torch.float16 else {}, scale_maxabs=True)
+
+    def quadratic(score, b, h, q_idx, kv_idx):
+        return score * score
+    q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 64, torch.float16))
+    with pytest.raises(NotImplementedError):
+        fa.flax_attention(q, k, v, score_mod=quadratic)
