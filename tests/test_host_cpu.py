@@ -208,3 +208,28 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".cuh")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "from oracle" not in text, f
+
+
+def test_affine_score_mod_lowering_on_cpu():
+    """A callable that is affine in the score becomes dense tables; one that is not is refused."""
+    import torch
+    from flaxattention_amd.core.common import affine_score_mod
+    table = torch.randn(3, 9, generator=torch.Generator().manual_seed(1))
+
+    def rel_table(score, b, h, q_idx, kv_idx):
+        return score + table[h.long(), (q_idx - kv_idx).clamp(-4, 4).long() + 4]
+
+    def scaled(score, b, h, q_idx, kv_idx):
+        return torch.where(q_idx >= kv_idx, score * 0.5, score * 2.0) - 1.5 * b
+
+    s = affine_score_mod(rel_table, 2, 3, 6, 7, "cpu")
+    assert s.kind == _lib.SCORE_AFFINE and s.mul is None and tuple(s.add.shape) == (1, 3, 6, 7)
+    c = s.c_struct()
+    assert (c.stride_b, c.stride_h, c.stride_q) == (0, 42, 7) and c.mul is None and c.add == s.add.data_ptr()
+    q, kv = torch.arange(6).reshape(6, 1), torch.arange(7).reshape(1, 7)
+    assert torch.equal(s.add[0, 2], table[2][(q - kv).clamp(-4, 4) + 4])
+    s = affine_score_mod(scaled, 2, 3, 6, 7, "cpu")
+    assert tuple(s.mul.shape) == (2, 1, 6, 7) and torch.equal(s.mul[1, 0], torch.where(q >= kv, 0.5, 2.0))
+    assert torch.equal(s.add[1, 0], torch.full((6, 7), -1.5))
+    assert affine_score_mod(lambda sc, b, h, q_, k_: sc * sc, 1, 1, 4, 4, "cpu") is None
+    assert affine_score_mod(lambda sc, b, h, q_, k_: sc + 0.0 * q_, 1, 1, 4, 4, "cpu").kind == _lib.SCORE_IDENTITY
