@@ -153,6 +153,13 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
     // doing both blocks side by side
 #pragma unroll
     for (int nb = 0; nb < BN / 32; nb++) {
+      // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
+      // entirely hidden (nothing to do)
+      int cls = kBlockAll;
+      if (masked) {
+        cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        if (cls == kBlockNone) continue;
+      }
       // dP starts at -delta, so the accumulator comes out as dP - delta
       float16_t sacc, dpacc, gacc;
 #pragma unroll
@@ -177,7 +184,7 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
           gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
         }
       }
-      if (masked) {
+      if (cls == kBlockMixed) {
         // a real branch whose inputs pass through the asm, so that none of the mask
         // arithmetic can be hoisted into the unmasked path
         int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
@@ -262,7 +269,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
-  const int wk = w;  // key block (32 rows) of this wave
+  const int wk = __builtin_amdgcn_readfirstlane(w);  // key block (32 rows) of this wave (wave-uniform)
   const int nkt = (p.Lkv + BN - 1) / BN;
   int kt, bh;  // early key tiles see the most queries under causal masks
   xcd_tile_map(blockIdx.x, nkt, p.Hkv * p.B, kt, bh);
@@ -387,6 +394,11 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       for (int qs = 0; qs < QBW; qs++) {
       // ---- S = Q.K^T and dP = dO.V^T for 32 query rows x 32 keys ----
       const int qrow_w = qs * 32;
+      int cls = kBlockAll;
+      if (masked) {
+        cls = band_block_class(p.mask, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
+        if (cls == kBlockNone) continue;
+      }
       float16_t sacc, dpacc;
       const int ql = qrow_w + 4 * g;  // local row of register 0
 #pragma unroll
@@ -424,7 +436,11 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
           }
         }
       }
-      if (masked) mask_block_kv(sacc, p.mask, visible, q0 + ql, kv_col, p.Lq, p.Lkv);
+      if (cls == kBlockMixed) {
+        int q_opaque = q0 + ql, kv_opaque = kv_col;
+        asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));  // keeps the mask arithmetic behind this branch
+        mask_block_kv(sacc, p.mask, visible, q_opaque, kv_opaque, p.Lq, p.Lkv);
+      }
       vec8 pf[2], dsf[2];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {

@@ -5,28 +5,26 @@
 // for 16-bit inputs, with a real online softmax and with skipping of masked-out
 // KV tiles, which the reference computes but never uses.
 //
-// Work decomposition: one workgroup (4 waves) per BM query rows of one (batch,
-// head); each wave owns RQ blocks of 32 query rows (RQ = 2, BM = 256 for D = 64;
-// RQ = 1, BM = 128 for D = 128).  KV tiles of 64 rows go through two LDS stages
-// (register-prefetched one tile ahead, one workgroup barrier per tile).  Every K
-// and V fragment read from LDS feeds RQ MFMAs, and every K/V tile fetched from L2
-// serves BM query rows: with 128 B rows (D = 64) the kernel is otherwise bound by
-// L2->LDS and LDS->register traffic long before the matrix cores are busy.
-// Per 32-key step and wave:
-//   S^T[kv, q]  = K_step . Q^T          4 x RQ v_mfma_f32_32x32x16 (D = 64)
+// Two kernels.  fwd_mfma_kernel (any supported D, tile lists or not): one workgroup
+// (4 waves) per 128 query rows of one (batch, head), one 32-row block per wave; KV tiles of
+// 64 rows go through two LDS stages (register-prefetched one tile ahead, one workgroup
+// barrier per tile).  fwd_pipe_kernel (D = 64 without tile lists): 256 query rows per
+// workgroup, two blocks per wave, software-pipelined (see there).
+// Per 32-key step and 32-row block:
+//   S^T[kv, q]  = K_step . Q^T          D/16 v_mfma_f32_32x32x16
 //   online softmax in the accumulator layout: a lane holds 16 of the 32 scores
 //   of ONE query row, the other 16 sit in lane ^ 32 -> row max/sum are
 //   in-register reductions plus one permlane32 swap; the reference maximum only
 //   moves when it is beaten by 2^8, so the accumulator is rarely rescaled
-//   O^T[d, q] += V_step^T . P^T         4 x RQ v_mfma (P^T is already in B-operand
+//   O^T[d, q] += V_step^T . P^T         D/16 v_mfma (P^T is already in B-operand
 //   layout; V^T fragments come from transposing LDS reads)
 #include "mfma_common.cuh"
 
 namespace flex {
 
 constexpr int kFwdBN = 64;
-__host__ __device__ constexpr int fwd_rq(int D) { return D == 64 ? 2 : 1; }
-__host__ __device__ constexpr int fwd_bm(int D) { return 4 * 32 * fwd_rq(D); }
+constexpr int kFwdBM = 128;   // query rows of a list-driven workgroup = q granularity of the forward lists
+constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dense kernel (D = 64, no lists)
 
 template <typename T, int D, int KIND, bool ROUND_S>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
@@ -34,7 +32,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
                                                            T* __restrict__ o, float* __restrict__ lse2) {
   typedef typename Frag<T>::vec8 vec8;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int RQ = fwd_rq(D), BM = fwd_bm(D), BN = kFwdBN;
+  constexpr int RQ = 1, BM = kFwdBM, BN = kFwdBN;
   constexpr int DS = D / 16;     // k-steps of the Q.K^T product
   constexpr int DB = D / 32;     // 32-row blocks of O^T
   constexpr int ROWE = D + 8;    // LDS row length in elements (16 B of padding)
@@ -196,7 +194,11 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
           // can be hoisted above the branch
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-          mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+          // most 32x32 blocks of a partial tile are entirely visible or entirely hidden
+          const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
+                                           __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
+          if (cls == kBlockNone) fill_masked(sacc[a]);
+          else if (cls == kBlockMixed) mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
       }
       // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
@@ -299,9 +301,8 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
                                                            T* __restrict__ o, float* __restrict__ lse2) {
   typedef typename Frag<T>::vec8 vec8;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int D = 64, RQ = 2, BM = fwd_bm(D), BN = kFwdBN;
+  constexpr int D = 64, RQ = 2, BM = kPipeBM, BN = kFwdBN;
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
-  static_assert(fwd_rq(D) == RQ, "two query blocks per wave");
   __shared__ __align__(16) T Ksm[3][BN * ROWE];
   __shared__ __align__(16) T Vsm[3][BN * ROWE];
 
@@ -480,7 +481,11 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
           // arithmetic can be hoisted into the unmasked path
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-          mask_block_q(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+          // most 32x32 blocks of a partial tile are entirely visible or entirely hidden
+          const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
+                                           __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
+          if (cls == kBlockNone) fill_masked(s_cur);
+          else if (cls == kBlockMixed) mask_block_q(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
         // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
         float m_rel = xhalf_max(block_max(s_cur));
@@ -562,15 +567,18 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 
 template <typename T, int D, int KIND>
 static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
-  const int nqt = (p.Lq + fwd_bm(D) - 1) / fwd_bm(D);
-  dim3 grid(nqt * p.Hq * p.B);
-  if constexpr (D == 64) {
+  // D = 64 without tile lists (every workgroup has the same work): the pipelined kernel with
+  // 256-row workgroups.  With lists the 128-row kernel: twice the workgroups, half the length of the
+  // longest one, which is what bounds a causal-like schedule.
+  if (D == 64 && !p.tiles.kv_num) {
+    dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
     if (p.flags & FLEX_ROUND_S)
       hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
     else
       hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
     return;
   }
+  dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B);
   if (p.flags & FLEX_ROUND_S)
     hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
   else
@@ -609,14 +617,14 @@ bool flex_mfma_shape_ok(const FlexAttnParams& p) {
 // which: 0 = forward and decode lists, 1 = backward lists
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
   const bool ok = (dtype == FLEX_F16 || dtype == FLEX_BF16) && D == Dv && (D == 64 || D == 128);
-  *qb = !ok ? 0 : (which == 0 ? fwd_bm(D) : 128);
+  *qb = !ok ? 0 : 128;
   *kvb = !ok ? 0 : (which == 0 ? kFwdBN : 128);
 }
 
 bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
   if (!flex_mfma_shape_ok(p)) return false;
   const FlexTileLists& t = p.tiles;
-  return !t.kv_num || (t.q_block == fwd_bm(p.D) && t.kv_block == kFwdBN);
+  return !t.kv_num || (t.q_block == kFwdBM && t.kv_block == kFwdBN);
 }
 
 int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {

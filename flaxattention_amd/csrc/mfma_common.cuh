@@ -216,6 +216,25 @@ struct Mask2 {
 constexpr int kBig = 1 << 30;
 __device__ __forceinline__ int clamp_big(int x) { return min(max(x, -kBig), kBig); }
 
+// Wave-uniform classification of one 32-query x 32-key block under a band mask:
+// kBlockAll = every entry visible (no mask evaluation needed), kBlockNone = nothing visible,
+// kBlockMixed = evaluate per element.  q_first / kv_first are the block's first query row and
+// key (wave-uniform values).  Bitmap masks are always kBlockMixed.
+enum { kBlockMixed = 0, kBlockAll = 1, kBlockNone = 2 };
+__device__ __forceinline__ int band_block_class(const FlexMask& m, int q_first, int kv_first, int Lq, int Lkv) {
+  if (m.kind != FLEX_MASK_BAND) return kBlockMixed;
+  const int lo = clamp_big(m.lo), hi = clamp_big(m.hi), snk = clamp_big(m.sink);
+  const int q_last = q_first + 31, kv_last = kv_first + 31;
+  const int dmin = q_first + m.q_offset - kv_last, dmax = q_last + m.q_offset - kv_first;
+  if (dmin >= lo && (dmax <= hi || kv_last <= snk) && kv_last < Lkv && q_last < Lq) return kBlockAll;
+  if (dmax < lo || (dmin > hi && kv_first > snk) || kv_first >= Lkv || q_first >= Lq) return kBlockNone;
+  return kBlockMixed;
+}
+__device__ __forceinline__ void fill_masked(float16_t& x) {
+#pragma unroll
+  for (int r = 0; r < 16; r++) x[r] = -INFINITY;
+}
+
 // one 32-key block: register r holds key kv0 + 4*g + acc_row(r); lane owns query q
 __device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
                                              int Lkv) {

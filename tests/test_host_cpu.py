@@ -55,7 +55,7 @@ def test_workspace_and_tile_queries_without_gpu():
     assert L.flexattn_block_mask_workspace_bytes(2, 3, 4, 5) >= 2 * 2 * 3 * 4 * 5
     qb, kvb = ctypes.c_int32(), ctypes.c_int32()
     L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
-    assert (qb.value, kvb.value) == (256, 64)
+    assert (qb.value, kvb.value) == (128, 64)
     L.flexattn_preferred_tiles(_lib.FLEX_BF16, 128, 128, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (128, 64)
     L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 1, ctypes.byref(qb), ctypes.byref(kvb))
