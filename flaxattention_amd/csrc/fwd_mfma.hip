@@ -144,6 +144,11 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
     // Each 32-row half of the tile is one online-softmax step.
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
+      // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
+      // entirely hidden (the step is skipped)
+      int cls = kBlockAll;
+      if (masked) cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+      if (cls != kBlockNone) {
       // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
       vec8 kfr[DS], vfr[2][DB];
       {
@@ -187,18 +192,12 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
           sacc[a][r] = sm.apply_sub(s0, acc_row(r), m_use[a]);
           sacc[a][r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use[a]);
         }
-        if (masked) {
-          // a real branch: without the barrier the compiler evaluates the mask for every
-          // tile and selects, which costs as much as the softmax itself
-          // every input of the mask arithmetic passes through this asm, so that none of it
-          // can be hoisted above the branch
+        if (cls == kBlockMixed) {
+          // a real branch: every input of the mask arithmetic passes through this asm, so that
+          // none of it can be hoisted into the unmasked path (it costs as much as the softmax)
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-          // most 32x32 blocks of a partial tile are entirely visible or entirely hidden
-          const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
-                                           __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
-          if (cls == kBlockNone) fill_masked(sacc[a]);
-          else if (cls == kBlockMixed) mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+          mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
       }
       // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
@@ -248,6 +247,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 #pragma unroll
           for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
       }
+      }  // block not entirely hidden
       if (nb == 0 && it + 1 < nt) {
         // the other stage was last read before the previous barrier: refill it with the
         // tile prefetched into registers, then start fetching the one after
