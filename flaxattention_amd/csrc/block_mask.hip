@@ -32,6 +32,20 @@ __global__ __launch_bounds__(kClassifyThreads) void classify_tiles_kernel(
       uint32_t bits = visible.bits_bh[(int64_t)(q0 + r) * visible.stride_q + (kv0 >> 5) + w];
       cnt += __popc(bits);
     }
+  } else if (mask.kind == FLEX_MASK_BAND) {
+    // closed form per row: with d = q + q_offset - kv the visible keys of a row are
+    //   { kv <= U } minus the gap { S < kv < W },   U = q + q_offset - lo,  W = q + q_offset - hi,  S = sink
+    // (d >= lo <=> kv <= U;  d <= hi <=> kv >= W), so the count inside [kv0, kv_end] takes a few
+    // integer operations instead of kvb evaluations.  Same count as the element-wise loop below.
+    const long long kv_end = (long long)kv0 + kvb - 1;
+    for (int r = threadIdx.x; r < qb; r += kClassifyThreads) {
+      const long long qo = (long long)q0 + r + mask.q_offset;
+      const long long top = min(qo - mask.lo, kv_end);           // last visible candidate in the tile
+      const long long seen = max(0LL, top - kv0 + 1);
+      const long long gap_lo = max((long long)mask.sink + 1, (long long)kv0);
+      const long long gap_hi = min(qo - mask.hi - 1, top);
+      cnt += (unsigned long long)(seen - max(0LL, gap_hi - gap_lo + 1));
+    }
   } else {
     for (long long t = threadIdx.x; t < total; t += kClassifyThreads) {
       int r = (int)(t / kvb), c = (int)(t % kvb);

@@ -109,3 +109,26 @@ def test_from_kv_blocks_transposes(dev):
                                       mask_mod=bm.mask_mod)
     for f in ["q_num_blocks", "q_indices", "full_q_num_blocks", "full_q_indices"]:
         assert torch.equal(getattr(bm, f), getattr(bm2, f)), f
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_band_closed_form_matches_brute_force(dev, seed):
+    """Band masks are classified per tile from a closed-form row count; the oracle evaluates every
+    (q, kv) pair.  Random band parameters, including unbounded sides, sinks and offsets."""
+    import random
+    from flaxattention_amd.core.common import INT_MAX
+    rnd = random.Random(50 + seed)
+    Q, KV = rnd.choice([(256, 384), (300, 200), (512, 512), (64, 1000)])
+    lo = rnd.choice([INT_MIN, 0, -17, 5, 130])
+    hi = rnd.choice([INT_MAX, 10, 128, 333, max(lo, 0) + 40])
+    sink = rnd.choice([-1, 0, 3, 127, 200])
+    off = rnd.choice([0, 0, KV - Q, 13])
+    bs = rnd.choice([128, 64, (128, 64)])
+    print(f"band lo={lo} hi={hi} sink={sink} off={off} Q{Q} KV{KV} bs{bs}", flush=True)
+    mask = MaskMod(lo, hi, sink, off, name="band")
+
+    def omask(b, h, q_idx, kv_idx):
+        d = q_idx + off - kv_idx
+        return (d >= lo) & ((d <= hi) | (kv_idx <= sink))
+    bm = fa.create_block_mask(mask, 1, 2, Q, KV, BLOCK_SIZE=bs, device=dev)
+    check(bm, ref_create_block_mask(omask, 1, 2, Q, KV, BLOCK_SIZE=bs))
