@@ -52,7 +52,7 @@ class FlexAttnParams(C.Structure):
                 ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
                 ("scale", C.c_float), ("flags", C.c_int32),
                 ("score", FlexScoreMod), ("mask", FlexMask), ("tiles", FlexTileLists),
-                ("tiles_bwd", FlexTileLists)]
+                ("tiles_bwd", FlexTileLists), ("q_index_base", C.c_int32), ("pad_", C.c_int32)]
 
 
 EXPORTS = [

@@ -95,10 +95,13 @@ class _Plan:
         self.lists_bwd = None   # tile lists for the backward kernels
         self.keep = [mask.bits, score.mul, score.add]
 
-    def params(self, q, k, v, o) -> _lib.FlexAttnParams:
+    def params(self, q, k, v, o, q_index_base: int = 0) -> _lib.FlexAttnParams:
+        """q / o may be a slice of rows [q_index_base, q_index_base + q.shape[2]) of the planned query
+        (decode in chunks); everything else refers to the whole problem."""
         p = _lib.FlexAttnParams()
         p.dtype = _DTYPES[self.dtype]
-        p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = self.B, self.Hq, self.Hkv, self.Lq, self.Lkv, self.D, self.Dv
+        p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = self.B, self.Hq, self.Hkv, q.shape[2], self.Lkv, self.D, self.Dv
+        p.q_index_base = int(q_index_base)
         for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
             if t.stride(3) != 1:
                 raise _lib.FlexAttnError("the feature axis must be contiguous")
@@ -165,13 +168,20 @@ def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
     want = opts.get("decode")
     if want is False:
         return 0
-    Hq, Lq, D = q.shape[1], q.shape[2], q.shape[3]
-    fits = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
-            and (Hq // k.shape[1]) * Lq <= 64 and score.kind != _lib.SCORE_AFFINE
-            and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
+    B, Hq, Lq, D = q.shape
+    G = Hq // k.shape[1]
+    ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
+          and score.kind != _lib.SCORE_AFFINE and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
     if want is True:
         return -1   # the library reports what does not fit
-    return -1 if fits and k.shape[2] >= 512 else 0
+    if not ok:
+        return 0
+    if G * Lq <= 64:
+        return -1 if k.shape[2] >= 512 else 0
+    # 65..256 rows against a long KV cache: a few decode passes over the cache beat a forward grid
+    # that would leave most compute units without a workgroup (one per 128 query rows and head)
+    few_workgroups = B * Hq * ((Lq + 127) // 128) < 256
+    return -1 if (G == 1 and Lq <= 256 and k.shape[2] >= 4096 and few_workgroups) else 0
 
 
 _holders: dict = {}
@@ -204,11 +214,28 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     with torch.cuda.device(q.device):
         if plan.decode_splits != 0:
             splits = max(plan.decode_splits, 0)   # 0 asks the library for its default
-            nbytes = L.flexattn_decode_workspace_bytes(p, splits)
-            ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
-            rc = L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(),
-                                   splits, ws.data_ptr(), _stream(q))
-            _lib.check(rc, "flexattn_decode")
+            rows = max(64 // (plan.Hq // plan.Hkv), 1)   # query rows one decode call takes
+            if plan.Lq <= rows:
+                chunks = [(0, plan.Lq, q, o, lse2, p)]
+            else:
+                # a longer query goes through the decode kernel 64 rows at a time (rows is 64 here:
+                # chunking is only chosen without GQA packing), each call seeing its row offset
+                chunks = []
+                for s0 in range(0, plan.Lq, rows):
+                    s1 = min(s0 + rows, plan.Lq)
+                    qc, oc = q[:, :, s0:s1], o[:, :, s0:s1]
+                    lc = torch.empty((plan.B, plan.Hq, s1 - s0), dtype=torch.float32, device=q.device)
+                    chunks.append((s0, s1, qc, oc, lc, plan.params(qc, k, v, oc, q_index_base=s0)))
+            ws = None
+            for s0, s1, qc, oc, lc, pc in chunks:
+                nbytes = L.flexattn_decode_workspace_bytes(pc, splits)
+                if ws is None or ws.numel() < nbytes:
+                    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=q.device)
+                rc = L.flexattn_decode(pc, qc.data_ptr(), k.data_ptr(), v.data_ptr(), oc.data_ptr(), lc.data_ptr(),
+                                       splits, ws.data_ptr(), _stream(q))
+                _lib.check(rc, "flexattn_decode")
+                if lc is not lse2:
+                    lse2[:, :, s0:s1] = lc
         else:
             rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), None, _stream(q))
             _lib.check(rc, "flexattn_fwd")

@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   const int32_t* part_idx = nullptr;
   int n_full = 0, steps_total;
   if (tl.kv_num && G == 1) {
-    const int64_t row = (b * tl.stride_b + hk * tl.stride_h) * tl.n_q_blocks;
+    const int64_t row = (b * tl.stride_b + hk * tl.stride_h) * tl.n_q_blocks + p.q_index_base / tl.q_block;
     n_full = tl.full_kv_num[row];
     const int n_part = tl.kv_num[row];
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     for (int nb = 0; nb < NB; nb++) {
       float16_t sacc = nb ? s_b : s_a;
       const float m_use = (m_run[nb] == -INFINITY) ? 0.f : m_run[nb];
-      sm[nb].tile(col_q[nb], kv0 + 4 * g);
+      sm[nb].tile(col_q[nb] + p.q_index_base, kv0 + 4 * g);
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float s0 = sacc[r], s1 = sacc[r + 1];
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
       if (need_mask) {
         // a real branch whose inputs pass through the asm, so that none of the mask
         // arithmetic can be hoisted into the unmasked path
-        int q_opaque = col_q[nb], kv_opaque = kv0;
+        int q_opaque = col_q[nb] + p.q_index_base, kv_opaque = kv0;
         asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
         Mask2 visible(p.mask, b, col_h[nb], p.Lkv);
         mask_block_q(sacc, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);

@@ -50,7 +50,7 @@ static int validate(const FlexAttnParams* p, const char* who) {
     const FlexTileLists& t = *both[i];
     if (!t.kv_num) continue;
     if (!t.kv_idx || !t.full_kv_num || !t.full_kv_idx) { flex_set_error("%s: tile lists need kv_idx, full_kv_num and full_kv_idx", who); return 1; }
-    if (t.q_block <= 0 || t.kv_block <= 0 || (int64_t)t.n_q_blocks * t.q_block < p->Lq || (int64_t)t.n_kv_blocks * t.kv_block < p->Lkv) {
+    if (t.q_block <= 0 || t.kv_block <= 0 || (int64_t)t.n_q_blocks * t.q_block < (int64_t)p->Lq + p->q_index_base || (int64_t)t.n_kv_blocks * t.kv_block < p->Lkv) {
       flex_set_error("%s: tile lists (%d x %d blocks of %d x %d) do not cover Lq=%d, Lkv=%d", who, t.n_q_blocks, t.n_kv_blocks, t.q_block, t.kv_block, p->Lq, p->Lkv);
       return 1;
     }
@@ -80,6 +80,7 @@ extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) { return
 extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                             void* workspace, flexattn_stream_t stream) {
   if (int rc = validate(p, "flexattn_fwd")) return rc;
+  if (p->q_index_base != 0) { flex_set_error("flexattn_fwd: q_index_base is for flexattn_decode only"); return 1; }
   if (!q || !k || !v || !o) { flex_set_error("flexattn_fwd: null tensor pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
@@ -102,6 +103,7 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
                             const float* lse2, const void* d_o, void* dq, void* dk, void* dv, void* workspace,
                             flexattn_stream_t stream) {
   if (int rc = validate(p, "flexattn_bwd")) return rc;
+  if (p->q_index_base != 0) { flex_set_error("flexattn_bwd: q_index_base is for flexattn_decode only"); return 1; }
   if (!q || !k || !v || !o || !lse2 || !d_o || !dq || !dk || !dv || !workspace) { flex_set_error("flexattn_bwd: null pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
@@ -120,6 +122,7 @@ extern "C" size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32
 extern "C" int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                                int32_t num_splits, void* workspace, flexattn_stream_t stream) {
   if (int rc = validate(p, "flexattn_decode")) return rc;
+  if (p->q_index_base < 0 || p->q_index_base % 64 != 0) { flex_set_error("flexattn_decode: q_index_base must be a non-negative multiple of 64 (got %d)", p->q_index_base); return 1; }
   if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
   if (!flex_decode_supported(*p)) {
     flex_set_error("flexattn_decode: needs fp16/bf16, D == Dv in {64,128}, Lq <= 64 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);

@@ -121,6 +121,12 @@ typedef struct FlexAttnParams {
   FlexMask mask;
   FlexTileLists tiles;     /* lists for flexattn_fwd / flexattn_decode */
   FlexTileLists tiles_bwd; /* lists for flexattn_bwd (its kernels tile differently) */
+  /* flexattn_decode only (0 elsewhere): the query tensor passed in is rows
+   * [q_index_base, q_index_base + Lq) of a longer query; score_mod, mask_mod and the tile
+   * lists see the full-sequence row index.  Lets a caller run a query of more than 64 rows
+   * against a long KV cache as several decode calls.  A multiple of 64. */
+  int32_t q_index_base;
+  int32_t pad_;
 } FlexAttnParams;
 
 int flexattn_abi_version(void);

@@ -98,3 +98,24 @@ def test_decode_is_chosen_automatically(dev):
     assert max_abs(a.detach().cpu(), b.cpu()) <= 2e-3
     a.sum().backward()
     assert torch.isfinite(qg.grad).all() and qg.grad.abs().max() > 0
+
+
+def test_decode_in_chunks_of_64_rows(dev):
+    """Queries of 65..256 rows against a long KV cache run as several decode calls, each seeing its
+    row offset in score_mod, mask_mod and the tile lists (ALiBi + offset-causal, ragged last chunk)."""
+    from flaxattention_amd.core.attention import _make_plan
+    B, H, Lq, Lkv, D = 1, 2, 160, 4096, 64
+    q, k, v = seeded_qkv(B, H, H, Lq, Lkv, D, torch.float16)
+    mask, omask = offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq)
+    bm = fa.create_block_mask(mask, B, H, Lq, Lkv, device=dev)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, None).decode_splits < 0          # chosen automatically
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, {"decode": False}).decode_splits == 0
+    out, lse = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True)
+    want, want_lse = ref_attention(q, k, v, o_alibi_config(H), omask, strict=True, return_lse=True)
+    a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
+    print(f"  chunked decode O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
+    assert a <= 2e-2 and r <= 1e-3
+    assert max_abs(lse.cpu(), want_lse) <= 2e-2
+    ref = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, kernel_options={"decode": False})
+    assert max_abs(out.cpu(), ref.cpu()) <= 2e-3
