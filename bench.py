@@ -234,6 +234,15 @@ def pmc_probe(dev, name, opts):
         pr.bwd("dq")
         pr.bwd("dkv")
     torch.cuda.synchronize()
+    # configuration 5: the decode kernels at q_len 1 and 64 (KV 16384), three launches each
+    from flaxattention_amd.masks import offset_causal_mask
+    from flaxattention_amd.mods import generate_alibi_bias
+    for ql, splits in ((1, 12), (64, 8)):
+        pd = Prepared(dev, torch.float16, 8, 8, 8, ql, 16384, 64, generate_alibi_bias(8, -1.0), offset_causal_mask(16384 - ql),
+                      decode_splits=splits)
+        for _ in range(3):
+            pd.decode()
+    torch.cuda.synchronize()
 
 
 def run_mfma_probe(dev):
