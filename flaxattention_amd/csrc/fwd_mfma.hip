@@ -294,6 +294,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 // unit u never touches an accumulator that a matrix instruction is writing.
 // KV tiles go through three LDS stages with one workgroup barrier per tile: a
 // stage is refilled only after a barrier that follows its last fragment read.
+// Tiles are fetched global -> LDS directly (no staging registers, no LDS stores),
+// one tile ahead of the one being read.
 // ---------------------------------------------------------------------------
 template <typename T, int KIND, bool ROUND_S>
 __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, const T* __restrict__ q,
@@ -302,9 +304,15 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   typedef typename Frag<T>::vec8 vec8;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int D = 64, RQ = 2, BM = kPipeBM, BN = kFwdBN;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
-  __shared__ __align__(16) T Ksm[3][BN * ROWE];
-  __shared__ __align__(16) T Vsm[3][BN * ROWE];
+  constexpr int DS = D / 16, DB = D / 32;
+  // KV tiles land in LDS straight from global memory (global_load_lds, 16 bytes per lane, a wave
+  // instruction fills 8 rows of 128 bytes), so rows are unpadded; the 16-byte chunk c of row r is
+  // kept at chunk position c ^ (r & 7), which makes both the row-fragment reads and the
+  // transposing reads conflict-free.  The lane that fills position (r, pos) therefore fetches
+  // chunk pos ^ (r & 7) of that row.
+  constexpr int kTileElems = BN * D;  // 8 KB per tile
+  __shared__ __align__(16) T Ksm[3][kTileElems];
+  __shared__ __align__(16) T Vsm[3][kTileElems];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -347,37 +355,50 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
-  u32x4 kreg[NLD], vreg[NLD];
-  auto load_tile = [&](int kv0) {
+  // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
+  const int fill_row = lane >> 3;                         // row inside the 8-row group = (row & 7)
+  const int fill_chunk = (lane & 7) ^ fill_row;           // logical chunk this lane fetches
+  auto issue_tile = [&](int stage, int kv0) {
+    const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      const int kvc = min(kv0 + r, p.Lkv - 1);
-      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
-      vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+    for (int j = 0; j < 2; j++) {
+      const int r0 = 16 * w + 8 * j;
+      const int row = min(r0 + fill_row, lim);
+      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + fill_chunk * 8;
+      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + fill_chunk * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
     }
   };
-  auto store_tile = [&](int stage) {
-#pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
-      *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
-    }
-  };
+  // ---- fragment reads ----
   vec8 kfr[DS], vfr[2][DB], pf[2];
-  auto read_k = [&](const T* Ks, int nb) {
-    const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+  int koff[DS];  // element offsets of this lane's K row fragments inside a 32-row block
 #pragma unroll
-    for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+  for (int s = 0; s < DS; s++) koff[s] = i32 * D + (((2 * s + g) ^ (i32 & 7)) * 8);
+  auto read_k = [&](const T* Ks, int nb) {
+#pragma unroll
+    for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(Ks + nb * 32 * D + koff[s]);
   };
+  // transposing reads: lane points at 4 elements of row 4g + (i16 >> 2) (+16tt, +8), logical column
+  // 32db + 16h + 4(i16 & 3)
+  int voff[DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
+#pragma unroll
+    for (int db = 0; db < DB; db++) {
+      const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+      voff[db] = rl * D + ((chunk ^ (rl & 7)) * 8) + 4 * (i16 & 1);
+    }
+  }
   auto read_v = [&](const T* Vs, int nb) {
 #pragma unroll
     for (int tt = 0; tt < 2; tt++)
 #pragma unroll
       for (int db = 0; db < DB; db++) {
-        const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-        vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+        const T* vp = Vs + (32 * nb + 16 * tt) * D + voff[db];
+        vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * D));
       }
   };
 
@@ -407,12 +428,11 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 
   constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
   int t_cur = nt > 0 ? tile_at(0) : 0;
-  int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) {
-    load_tile(t_cur * BN);
-    store_tile(0);
-  }
-  if (nt > 1) load_tile(t_nxt * BN);
+  int t_nxt = nt > 1 ? tile_at(1) : 0;   // tile it + 1
+  int t_nx2 = nt > 2 ? tile_at(2) : 0;   // tile it + 2
+  if (nt > 0) issue_tile(0, t_cur * BN);
+  if (nt > 1) issue_tile(1, t_nxt * BN);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   // S of the first unit
   read_k(Ksm[0], 0);
@@ -439,20 +459,23 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
     const T* Ks = Ksm[st];
     const T* Vs = Vsm[st];
     const T* Kn = Ksm[st_n];
+    const int st_p = st == 0 ? 2 : st - 1;  // stage of the previous tile = stage of tile it + 2
+    const int kv_nx2 = t_nx2 * BN;
     t_cur = t_nxt;
-    if (it + 2 < nt) t_nxt = tile_at(it + 2);
+    t_nxt = t_nx2;
+    if (it + 3 < nt) t_nx2 = tile_at(it + 3);
 #pragma unroll
     for (int nb = 0; nb < 2; nb++) {
 #pragma unroll
       for (int a = 0; a < RQ; a++) {
         const int q_row = q_row0 + 32 * a;
-        if (nb == 0 && a == 1 && it + 1 < nt) {
-          // stage st_n held the tile before the previous one; its last reads came before the
-          // previous barrier.  Refill it from the prefetch registers and fetch the tile after.
-          store_tile(st_n);
-          if (it + 2 < nt) load_tile(t_nxt * BN);
+        if (nb == 1 && a == 0) {
+          // this wave's share of tile it + 1 has landed; after the barrier everyone's has, and
+          // the previous tile's stage (last read before this barrier) can take tile it + 2
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+          if (it + 2 < nt) issue_tile(st_p, kv_nx2);
         }
-        if (nb == 1 && a == 0) __syncthreads();  // the next tile's stage is complete
         if (a == 1) read_v(Vs, nb);              // V columns of this step, first used in region B
 
         // ---- region A: S^T of the next unit || score_mod relative to the running reference max ----
