@@ -262,6 +262,26 @@ def run_mfma_probe(dev):
     return flops.value / us / 1e6
 
 
+def run_mix_probe(dev):
+    """Matrix flop rate of the library's instruction-mix probe: 8, 12 or 16 MFMAs interleaved with the vector work of
+    one 32x32 score block (80 FMAs + 16 exponentials), two waves per SIMD.  The ceiling of a fused attention step of
+    that mix on this GPU: 8 = forward at D 64, 12 = dQ kernel, 16 = dK/dV kernel and forward at D 128."""
+    from flaxattention_amd import _lib
+    L = _lib.lib()
+    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
+    flops = C.c_double(0.0)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    out = {}
+    for nm in (8, 12, 16):
+        def go():
+            rc = L.flexattn_probe_mix(sink.data_ptr(), 2048, nm, C.byref(flops), stream)
+            if rc:
+                _lib.check(rc, "flexattn_probe_mix")
+        us = event_time_us(go, 20)
+        out[str(nm)] = round(flops.value / us / 1e6, 1)
+    return out
+
+
 def run_block_mask_build(dev):
     """create_block_mask for the masks of configurations 3 and 4 at the API's block size 128 (device time of
     the classify / order kernels plus the front end's enqueue cost; the reference builds it outside its timed loop)."""
@@ -345,6 +365,9 @@ def main():
         probe = run_mfma_probe(dev)
         log(f"MFMA-only probe kernel (fp16, pseudo-random operands): {probe:.0f} TFLOP/s sustained")
         extra["mfma_probe_tflops"] = round(probe, 1)
+        mix = run_mix_probe(dev)
+        log(f"instruction-mix probe (MFMAs per 96 vector instructions -> matrix TFLOP/s): {mix}")
+        extra["mix_probe_tflops"] = mix
         bmb = run_block_mask_build(dev)
         log(f"create_block_mask: {bmb} us")
         extra["block_mask_build_us"] = bmb

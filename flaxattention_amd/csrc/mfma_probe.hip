@@ -36,6 +36,59 @@ __global__ __launch_bounds__(256, 2) void mfma_probe_kernel(float* __restrict__ 
   sink[blockIdx.x * 256 + threadIdx.x] = s;
 }
 
+// Second aid: the instruction mix of a fused attention step.  Per "unit" a wave issues NM
+// matrix instructions interleaved with 80 fused multiply-adds and 16 exponentials on 16
+// registers (what scaling, score_mod, exp, rounding and row sums cost per 32x32 score block),
+// two waves per SIMD.  NM = 8 is the forward at D = 64, 12 the dQ kernel, 16 the dK/dV kernel
+// or the forward at D = 128.  Its rate is the ceiling of that mix on this GPU: matrix and
+// vector instructions share the issue port and the power budget.
+template <int NM>
+__global__ __launch_bounds__(256, 2) void mix_probe_kernel(float* __restrict__ sink, int iters, float c0, float c1) {
+  float16_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[j][i] = 0.f;
+  half8_t a[4], b[4];
+  unsigned x = (blockIdx.x * 256u + threadIdx.x) * 2654435761u + 12345u;
+#pragma unroll
+  for (int s = 0; s < 4; s++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      x = x * 1664525u + 1013904223u;
+      a[s][e] = (_Float16)((float)((x >> 9) & 2047) * (1.f / 1024.f) - 1.f);
+      x = x * 1664525u + 1013904223u;
+      b[s][e] = (_Float16)((float)((x >> 9) & 2047) * (1.f / 1024.f) - 1.f);
+    }
+  float y[16];
+#pragma unroll
+  for (int r = 0; r < 16; r++) y[r] = (float)a[r & 3][r >> 2];
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int m = 0; m < NM; m++) acc[m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[m & 3], b[(m >> 2) & 3], acc[m & 3], 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 5; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) y[r] = __builtin_fmaf(y[r], c0, c1);
+#pragma unroll
+    for (int r = 0; r < 16; r++) y[r] = fast_exp2(y[r]);
+#pragma unroll
+    for (int m = 0; m < NM; m++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 80 / NM, 0);
+      __builtin_amdgcn_sched_group_barrier(0x400, 16 / NM, 0);
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; j++)
+#pragma unroll
+    for (int i = 0; i < 16; i++) s += acc[j][i];
+#pragma unroll
+  for (int r = 0; r < 16; r++) s += y[r];
+  sink[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
 }  // namespace flex
 
 void flex_set_error(const char* fmt, ...);
@@ -47,5 +100,21 @@ extern "C" int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per
   if (flops_per_launch) *flops_per_launch = 512.0 * 4 * 8.0 * iters * 2.0 * 32 * 32 * 16;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { flex_set_error("flexattn_probe_mfma: launch failed: %s", hipGetErrorString(e)); return 2; }
+  return 0;
+}
+
+// Same grid; `iters` units of `mfma_per_unit` (8, 12 or 16) matrix instructions + 96 vector instructions per wave.
+extern "C" int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch, void* stream) {
+  if (!sink || iters <= 0 || (mfma_per_unit != 8 && mfma_per_unit != 12 && mfma_per_unit != 16)) {
+    flex_set_error("flexattn_probe_mix: needs a device buffer of 512*256 floats, iters > 0 and mfma_per_unit in {8, 12, 16}");
+    return 1;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  if (mfma_per_unit == 8) hipLaunchKernelGGL(flex::mix_probe_kernel<8>, dim3(512), dim3(256), 0, st, sink, iters, 0.999f, 0.001f);
+  else if (mfma_per_unit == 12) hipLaunchKernelGGL(flex::mix_probe_kernel<12>, dim3(512), dim3(256), 0, st, sink, iters, 0.999f, 0.001f);
+  else hipLaunchKernelGGL(flex::mix_probe_kernel<16>, dim3(512), dim3(256), 0, st, sink, iters, 0.999f, 0.001f);
+  if (flops_per_launch) *flops_per_launch = 512.0 * 4 * (double)mfma_per_unit * iters * 2.0 * 32 * 32 * 16;
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { flex_set_error("flexattn_probe_mix: launch failed: %s", hipGetErrorString(e)); return 2; }
   return 0;
 }

@@ -191,6 +191,16 @@ int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const
  * *flops_per_launch receives the flop count of one launch. */
 int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, flexattn_stream_t stream);
 
+/* Second measurement aid, also without counterpart in the reference: the instruction mix of a
+ * fused attention step.  Per unit a wave issues `mfma_per_unit` (8, 12 or 16) matrix
+ * instructions interleaved with 80 fused multiply-adds and 16 exponentials (the vector work of
+ * one 32x32 score block), two waves per SIMD, `iters` units per wave.  Its matrix flop rate is
+ * the ceiling of that mix on this GPU (matrix and vector instructions share the issue port and
+ * the power budget): 8 = forward at D 64, 12 = dQ kernel, 16 = dK/dV kernel or forward at D 128.
+ * `sink` as above; *flops_per_launch receives the matrix flop count of one launch. */
+int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch,
+                       flexattn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

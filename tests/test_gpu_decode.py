@@ -81,6 +81,13 @@ def test_mfma_probe_runs(dev):
     assert flops.value == 512 * 4 * 8 * 4 * 2 * 32 * 32 * 16
     assert torch.isfinite(sink).all()
     assert L.flexattn_probe_mfma(None, 4, None, None) != 0 and b"probe" in L.flexattn_last_error()
+    for nm in (8, 12, 16):
+        rc = L.flexattn_probe_mix(sink.data_ptr(), 3, nm, ctypes.byref(flops), torch.cuda.current_stream(dev).cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert flops.value == 512 * 4 * nm * 3 * 2 * 32 * 32 * 16
+        assert torch.isfinite(sink).all()
+    assert L.flexattn_probe_mix(sink.data_ptr(), 3, 7, None, None) != 0 and b"probe_mix" in L.flexattn_last_error()
 
 
 def test_decode_is_chosen_automatically(dev):
