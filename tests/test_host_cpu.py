@@ -233,3 +233,25 @@ def test_affine_score_mod_lowering_on_cpu():
     assert torch.equal(s.add[1, 0], torch.full((6, 7), -1.5))
     assert affine_score_mod(lambda sc, b, h, q_, k_: sc * sc, 1, 1, 4, 4, "cpu") is None
     assert affine_score_mod(lambda sc, b, h, q_, k_: sc + 0.0 * q_, 1, 1, 4, 4, "cpu").kind == _lib.SCORE_IDENTITY
+
+
+def test_utils_score_matrix_and_picture(tmp_path):
+    """flaxattention/utils.py:17-49, 58-139: dense post-mod scores / mask of one (batch, head) and its picture."""
+    from flaxattention_amd.utils import _name_to_title, create_score_mod, visualize_attention_scores
+    from flaxattention_amd.masks import causal_mask
+    from flaxattention_amd.mods import generate_alibi_bias
+    g = torch.Generator().manual_seed(3)
+    q, k = torch.randn(2, 4, 6, 8, generator=g), torch.randn(2, 4, 9, 8, generator=g)
+    alibi = generate_alibi_bias(4)
+    got = create_score_mod(q[1, 2], k[1, 2], alibi, None, batch_idx=1, head_idx=2)
+    assert got.shape == (1, 1, 6, 9)
+    qi, ki = torch.arange(6).view(6, 1), torch.arange(9).view(1, 9)
+    want = (q[1, 2] @ k[1, 2].T) / 8 ** 0.5 + (qi - ki) * 2.0 ** (-(2 + 1) * 8.0 / 4)   # mods/alibi.py:15-18
+    assert torch.allclose(got[0, 0], want, atol=1e-6)
+    m = create_score_mod(q[0, 0], k[0, 0], None, causal_mask)
+    assert m.dtype == torch.bool and torch.equal(m[0, 0], qi >= ki)
+    assert _name_to_title("causal_mask_demo") == "Causal Mask Demo"
+    visualize_attention_scores(q, k, mask_mod=causal_mask, name="m", path=tmp_path / "mask_picture", head_idx=1)
+    assert (tmp_path / "mask_picture.png").stat().st_size > 1000
+    with pytest.raises(AssertionError):
+        visualize_attention_scores(q, k)
