@@ -4,8 +4,9 @@
 // (flaxattention/kernel/attention.py:338-553) and of jax.grad through the dense
 // path.  P is recomputed from the saved base-2 log-sum-exp.  Two kernels:
 //
-//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 128
-//                  (the entries of the 128-granular backward lists).  Transposed products keep one query
+//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 128 (64 at D = 128;
+//                  the entries of the 128-granular backward lists), fetched global -> LDS
+//                  directly into two stages.  Transposed products keep one query
 //                  row per lane, so lse and delta are per-lane scalars:
 //                    S^T = K.Q^T,  dP^T = V.dO^T,  dS^T = P^T o (dP^T - delta) * g,
 //                    dQ^T += K^T.dS^T.
@@ -20,22 +21,26 @@
 namespace flex {
 
 constexpr int kBM = 128;     // query tile (list granularity)
-constexpr int kBN = 128;     // key tile staged per step by the dQ kernel
+constexpr int kBN = 128;     // key tile staged per step by the dQ kernel at D = 64 (half of it at D = 128)
 constexpr int kListBN = 128; // key granularity of the backward tile lists = key rows of a dK/dV workgroup
 
 template <typename T, int D, int KIND, bool ROUND_S>
-__global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
                                                       const T* __restrict__ d_o, T* __restrict__ dq,
                                                       float* __restrict__ delta_out) {
   typedef typename Frag<T>::vec8 vec8;
-  constexpr int BM = kBM, BN = kBN;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BN * CPR / 256;
-  // two LDS stages: while one tile is consumed the next one is written, so a
-  // single workgroup barrier per tile suffices
-  __shared__ __align__(16) T Ksm[2][BN * ROWE];
-  __shared__ __align__(16) T Vsm[2][BN * ROWE];
+  // keys staged per step: 128 at D = 64, 64 at D = 128, so that two stages of K and V are 64 KB
+  // either way and two workgroups (two waves per SIMD) share a compute unit
+  constexpr int BM = kBM, BN = D == 64 ? kBN : kBN / 2;
+  constexpr int DS = D / 16, DB = D / 32, CPR = D / 8;
+  constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
+  constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor
+  // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled
+  // rows): while one tile is consumed the next one lands, one workgroup barrier per tile
+  __shared__ __align__(16) T Ksm[2][BN * D];
+  __shared__ __align__(16) T Vsm[2][BN * D];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -95,25 +100,38 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  u32x4 kreg[NLD], vreg[NLD];
-  auto load_tile = [&](int kv0) {
+  // tile fetch: wave w fills rows [32w, 32w + 32) of the K and the V tile, RPI rows per instruction;
+  // the lane that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
+  const int fill_row = lane / CPR, fill_pos = lane % CPR;
+  auto issue_tile = [&](int stage, int kv0) {
+    const int lim = p.Lkv - 1 - kv0;  // rows past the end: clamped (finite filler, masked out below)
 #pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
-      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
-      vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+    for (int j = 0; j < NI; j++) {
+      const int r0 = (BN / 4) * w + RPI * j;
+      const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);  // the wave's first row is a multiple of 16
+      const int row = min(r0 + fill_row, lim);
+      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
+      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
     }
   };
-  auto store_tile = [&](int stage) {
+  // element offsets inside a 32-row block: row fragments (row i32, chunk 2s + g sits at (2s) ^ kz) and
+  // transposing reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
+  const int kz = g ^ lds_swz<D>(i32);
+  int toff[2][DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
 #pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
-      *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
-    }
-  };
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        toff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
+      }
+  }
 
   Score2<KIND> sm;
   sm.init(p.score, p.scale, h);
@@ -126,11 +144,8 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
 
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) {
-    load_tile(t_cur * BN);
-    store_tile(0);
-  }
-  if (nt > 1) load_tile(t_nxt * BN);
+  if (nt > 0) issue_tile(0, t_cur * BN);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   const float neg_delta = -delta;
   for (int it = 0; it < nt; it++) {
@@ -139,14 +154,11 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
     const T* Ks = Ksm[it & 1];
     const T* Vs = Vsm[it & 1];
     if (it + 1 < nt) {
-      // the other stage was last read before the previous barrier: refill it with the
-      // tile prefetched into registers, then start fetching the one after
-      store_tile((it + 1) & 1);
+      // the other stage was last read before the previous barrier: the next tile lands there
+      // while this one is consumed; the tile index after that is looked up a tile ahead
+      issue_tile((it + 1) & 1, t_nxt * BN);
       t_cur = t_nxt;
-      if (it + 2 < nt) {
-        t_nxt = tile_at(it + 2);
-        load_tile(t_nxt * BN);
-      }
+      if (it + 2 < nt) t_nxt = tile_at(it + 2);
     }
 
     // one 32-key block at a time (S, dP, softmax, dQ): half the accumulator registers of
@@ -164,12 +176,12 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
       float16_t sacc, dpacc, gacc;
 #pragma unroll
       for (int r = 0; r < 16; r++) { sacc[r] = 0.f; dpacc[r] = neg_delta; }
-      const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
-      const T* vp = Vs + (nb * 32 + i32) * ROWE + 8 * g;
+      const T* kp = Ks + (nb * 32 + i32) * D;
+      const T* vp = Vs + (nb * 32 + i32) * D;
 #pragma unroll
       for (int s = 0; s < DS; s++) {
-        sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + 16 * s), qf[s], sacc);
-        dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + 16 * s), dof[s], dpacc);
+        sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + (((2 * s) ^ kz) * 8)), qf[s], sacc);
+        dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + (((2 * s) ^ kz) * 8)), dof[s], dpacc);
       }
       // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
       sm.tile(q_row, kv0 + nb * 32 + 4 * g);
@@ -209,13 +221,15 @@ __global__ __launch_bounds__(256, D == 64 ? 2 : 1) void bwd_dq_kernel(FlexAttnPa
       for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const T* ktp = Ks + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-          short4_t lo = lds_read_tr(ktp);
-          short4_t hi = lds_read_tr(ktp + 8 * ROWE);
+          const T* ktp = Ks + (32 * nb + 16 * tt) * D;
+          short4_t lo = lds_read_tr(ktp + toff[0][db]);
+          short4_t hi = lds_read_tr(ktp + toff[1][db]);
           dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[tt], dqacc[db]);
         }
       }
     }
+    // this wave's share of the next tile has landed; after the barrier everyone's has
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
 

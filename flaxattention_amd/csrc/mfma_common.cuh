@@ -369,6 +369,16 @@ __device__ __forceinline__ float tile_max(const float16_t (&x)[2]) {
   return max3(max3(a, b, x[0][15]), x[1][15], x[1][15]);
 }
 
+// Unpadded LDS tiles filled by direct global -> LDS loads (a wave instruction writes 1 KB of
+// consecutive rows): the 16-byte chunk c of row r is kept at chunk position c ^ lds_swz<D>(r).
+// With 128-byte rows (D = 64) two rows span the 64 banks and r & 7 spreads both the
+// row-fragment reads (16 rows, one chunk column) and the transposing reads (4 rows x 2 chunks
+// per 16 lanes) over distinct banks; with 256-byte rows (D = 128) every row starts at bank 0 and
+// the swizzle is a bijection of r & 15 whose low rows differ in the high chunk bits.
+template <int D> __device__ __forceinline__ constexpr int lds_swz(int r) {
+  return D == 64 ? (r & 7) : (((r & 3) << 2) | ((r >> 2) & 3));
+}
+
 // XCD-aware, heavy-first workgroup map.  Hardware deals consecutive workgroup ids
 // round-robin to the 8 XCDs (each has its own L2) and starts them in id order as
 // slots free up.  Every XCD gets a contiguous share of the (batch, head) pairs, so
