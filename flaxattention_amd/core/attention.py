@@ -282,14 +282,21 @@ def math_attention(query: Array, key: Array, value: Array, score_mod: Callable, 
                    mask_mod_other_buffers: Tuple = (), use_pallas: bool = False) -> Tuple[Array, Array]:
     """attention.py:67-106: (output, base-2 logsumexp).  ``block_mask`` is the
     tuple BlockMask.as_tuple() gives; only its last entry (the mask_mod) is
-    read, as in the reference (attention.py:45).  Runs the faithful kernels."""
-    if score_mod_other_buffers or mask_mod_other_buffers:
-        raise NotImplementedError("captured buffers are not supported")
+    read, as in the reference (attention.py:45).  Runs the faithful kernels.
+    ``score_mod_other_buffers`` / ``mask_mod_other_buffers`` are handed to the mods as
+    trailing arguments (attention.py:22-23, 36-44)."""
+    mask_mod = block_mask[-1]
+    if score_mod_other_buffers:
+        inner_score, sbufs = score_mod, tuple(score_mod_other_buffers)
+        score_mod = lambda score, b, h, q_idx, kv_idx: inner_score(score, b, h, q_idx, kv_idx, *sbufs)  # noqa: E731
+    if mask_mod_other_buffers:
+        inner_mask, mbufs = mask_mod, tuple(mask_mod_other_buffers)
+        mask_mod = lambda b, h, q_idx, kv_idx: inner_mask(b, h, q_idx, kv_idx, *mbufs)  # noqa: E731
     _require_device(query, key, value)
     q, k, v = map(_as_kernel_layout, (query, key, value))
     opts = dict(kernel_options or {})
     opts.setdefault("strict", True)
-    plan = _make_plan(q, k, v, score_mod, None, block_mask[-1], scale, opts)
+    plan = _make_plan(q, k, v, score_mod, None, mask_mod, scale, opts)
     return _FlexAttention.apply(q, k, v, plan)
 
 

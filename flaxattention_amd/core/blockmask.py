@@ -320,13 +320,14 @@ def create_block_mask(mask_mod: _mask_mod_signature, B: Optional[int], H: Option
         KV_BLOCK_SIZE = BLOCK_SIZE
     else:
         Q_BLOCK_SIZE, KV_BLOCK_SIZE = BLOCK_SIZE
+    real = (Q_LEN, KV_LEN)
     if Q_LEN < 128:
         Q_BLOCK_SIZE = Q_LEN
     else:
         Q_LEN = _round_up_to_multiple(Q_LEN, Q_BLOCK_SIZE)
     KV_LEN = _round_up_to_multiple(KV_LEN, KV_BLOCK_SIZE)
     dev = _device(device)
-    spec = resolve_mask_mod(mask_mod, B, H, Q_LEN, KV_LEN, dev)
+    spec = resolve_mask_mod(mask_mod, B, H, Q_LEN, KV_LEN, dev, real=real)
     lists = build_lists(spec, B, H, Q_LEN // Q_BLOCK_SIZE, KV_LEN // KV_BLOCK_SIZE, Q_BLOCK_SIZE, KV_BLOCK_SIZE, dev)
     bm = BlockMask(lists["kv_num_blocks"], lists["kv_indices"], lists["full_kv_num_blocks"], lists["full_kv_indices"],
                    lists["q_num_blocks"], lists["q_indices"], lists["full_q_num_blocks"], lists["full_q_indices"],

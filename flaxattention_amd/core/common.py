@@ -186,9 +186,15 @@ def affine_score_mod(fn: Callable, B: int, H: int, Lq: int, Lkv: int, device) ->
     q = torch.arange(min(Lq, P), dtype=torch.int32).reshape(1, 1, 1, -1, 1)
     kv = torch.arange(min(Lkv, P + 2), dtype=torch.int32).reshape(1, 1, 1, 1, -1)
     shape = (5, b.numel(), H, q.numel(), kv.numel())
-    try:
-        out = torch.broadcast_to(torch.as_tensor(fn(s.expand(shape), b, h, q, kv)).to(torch.float32), shape)
-    except Exception:
+    out = None
+    for where in ("cpu", device):   # a callable that indexes tensors living on the device cannot take CPU indices
+        try:
+            sw, bw, hw, qw, kw = (t.to(where) for t in (s, b, h, q, kv))
+            out = torch.broadcast_to(torch.as_tensor(fn(sw.expand(shape), bw, hw, qw, kw)).to(torch.float32), shape).cpu()
+            break
+        except Exception:
+            continue
+    if out is None:
         return None
     a0, c0 = (out[4] - out[2]) / 2.5, out[2]
     if not torch.isfinite(out).all() or not torch.allclose(out, a0 * s + c0, rtol=1e-5, atol=1e-5):
@@ -347,22 +353,98 @@ def _pad128(n: int) -> int:
     return (n + 127) // 128 * 128
 
 
-def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device) -> torch.Tensor:
-    """Evaluate a Python mask_mod (or a five-argument score_mod, which masks
-    where it returns -inf: flaxattention/core/blockmask.py:307-315) over the
-    whole index grid with device tensors.  bool [B,H,Q,KV]."""
-    b = torch.arange(B, dtype=torch.int32, device=device).reshape(B, 1, 1, 1)
-    h = torch.arange(H, dtype=torch.int32, device=device).reshape(1, H, 1, 1)
-    q = torch.arange(Q, dtype=torch.int32, device=device).reshape(1, 1, Q, 1)
-    kv = torch.arange(KV, dtype=torch.int32, device=device).reshape(1, 1, 1, KV)
+def _eval_mask(fn: Callable, b, h, q, kv) -> torch.Tensor:
+    """fn on broadcastable int32 index tensors -> bool tensor (a five-argument score_mod masks where it
+    returns -inf: flaxattention/core/blockmask.py:307-315)."""
+    dev = q.device
     if _get_mod_type(fn) == _ModificationType.SCORE_MOD:
-        out = fn(torch.zeros(B, H, Q, KV, device=device), b, h, q, kv)
-        m = ~torch.isneginf(torch.as_tensor(out, device=device))
-    else:
-        m = fn(b, h, q, kv)
-        if not torch.is_tensor(m):
-            m = torch.tensor(bool(m), device=device)
-    return m.to(device=device, dtype=torch.bool)
+        shape = torch.broadcast_shapes(b.shape, h.shape, q.shape, kv.shape)
+        out = fn(torch.zeros(shape, device=dev), b, h, q, kv)
+        return ~torch.isneginf(torch.as_tensor(out, device=dev))
+    m = fn(b, h, q, kv)
+    if not torch.is_tensor(m):
+        m = torch.tensor(bool(m), device=dev)
+    return m.to(torch.bool)
+
+
+def _index_arithmetic_only(fn, depth: int = 0) -> bool:
+    """True when `fn` provably computes from its index arguments alone: everything it closes over, defaults to
+    or reads from its globals is a number, a string, a module or another such function.  Anything else (a
+    tensor, an array, an object that may hold one) makes it a mod that may look positions up in a buffer."""
+    import functools
+    import types
+
+    def plain(x) -> bool:
+        if x is None or isinstance(x, (bool, int, float, complex, str, bytes, types.ModuleType, type)):
+            return True
+        if isinstance(x, MaskMod):
+            return x.bits is None
+        if isinstance(x, (tuple, list, frozenset, set)):
+            return all(plain(y) for y in x)
+        if isinstance(x, dict):
+            return all(plain(y) for y in x.values())
+        if isinstance(x, (types.FunctionType, types.BuiltinFunctionType, functools.partial)):
+            return _index_arithmetic_only(x, depth + 1)
+        return False
+
+    if depth > 4:
+        return False
+    if isinstance(fn, MaskMod):
+        return fn.bits is None
+    if isinstance(fn, functools.partial):
+        return plain(fn.func) and plain(fn.args) and plain(fn.keywords)
+    if isinstance(fn, types.BuiltinFunctionType):
+        return True
+    code = getattr(fn, "__code__", None)
+    if code is None or getattr(fn, "__self__", None) is not None:
+        return False
+    seen = [c.cell_contents for c in (fn.__closure__ or ())]
+    seen += list(fn.__defaults__ or ()) + list((fn.__kwdefaults__ or {}).values())
+    seen += [fn.__globals__[n] for n in code.co_names if n in fn.__globals__]
+    return all(plain(x) for x in seen)
+
+
+def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device,
+                         real: Optional[Tuple[int, int]] = None) -> torch.Tensor:
+    """Evaluate a Python mask_mod (or a five-argument score_mod) over the index grid [0,Q) x [0,KV) with
+    device tensors.  bool, broadcastable to [B,H,Q,KV].
+
+    `real` = (Q_LEN, KV_LEN) when the grid is the padded one of the block-mask builder, which treats
+    positions past the end as if they were real (blockmask.py:440-444).  A mod that looks positions up in
+    captured tensors must never be handed such indices (an out-of-range index into a device tensor stops
+    the process, and torch accepts CPU index tensors for device tensors, so trying on the CPU first is no
+    protection): unless the mod provably computes from its index arguments alone, the part of the grid past
+    the real lengths is evaluated with indices clamped to the last real position, which is what an
+    out-of-range gather yields under XLA."""
+    def grid(where, qs, ks, clamp=False):
+        q = torch.arange(qs[0], qs[1], dtype=torch.int32, device=where).reshape(1, 1, -1, 1)
+        kv = torch.arange(ks[0], ks[1], dtype=torch.int32, device=where).reshape(1, 1, 1, -1)
+        if clamp:
+            q, kv = q.clamp(max=Qr - 1), kv.clamp(max=KVr - 1)
+        b = torch.arange(B, dtype=torch.int32, device=where).reshape(B, 1, 1, 1)
+        h = torch.arange(H, dtype=torch.int32, device=where).reshape(1, H, 1, 1)
+        return _eval_mask(fn, b, h, q, kv).to(device)
+
+    Qr, KVr = (Q, KV) if real is None else (min(real[0], Q), min(real[1], KV))
+    core = grid(device, (0, Qr), (0, KVr))
+    if Qr == Q and KVr == KV:
+        return core
+
+    clamp = not _index_arithmetic_only(fn)
+
+    def beyond(qs, ks):
+        return grid(device, qs, ks, clamp)
+    pieces = [(core, (0, Qr), (0, KVr))]
+    if Qr < Q:
+        pieces.append((beyond((Qr, Q), (0, KV)), (Qr, Q), (0, KV)))
+    if KVr < KV:
+        pieces.append((beyond((0, Qr), (KVr, KV)), (0, Qr), (KVr, KV)))
+    Bm = max(t.shape[0] if t.dim() == 4 else 1 for t, _, _ in pieces)
+    Hm = max(t.shape[1] if t.dim() == 4 else 1 for t, _, _ in pieces)
+    m = torch.zeros((Bm, Hm, Q, KV), dtype=torch.bool, device=device)
+    for t, (q0, q1), (k0, k1) in pieces:
+        m[:, :, q0:q1, k0:k1] = torch.broadcast_to(t, (Bm, Hm, q1 - q0, k1 - k0))
+    return m
 
 
 def _fit_band(m2: torch.Tensor) -> Optional[MaskMod]:
@@ -408,12 +490,13 @@ def pack_bits(mask: torch.Tensor) -> torch.Tensor:
     return words.to(torch.int32).contiguous()
 
 
-def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, device) -> MaskMod:
+def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, device,
+                     real: Optional[Tuple[int, int]] = None) -> MaskMod:
     """Lower a mask_mod callable to a kernel functor that is exact on the
     index range [0, pad128(Q)) x [0, pad128(KV)).  Tagged functors pass
     through; any other callable is evaluated densely on the device once and
     either recognised as a band mask (checked against every entry) or kept as
-    a packed bitmap."""
+    a packed bitmap.  `real` gives the true sequence lengths when Q / KV are already rounded up."""
     if fn is None:
         return MaskMod(name="noop_mask")
     if isinstance(fn, MaskMod) and fn.bits is None:
@@ -424,7 +507,7 @@ def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, de
             return fn
         fn = fn.fn
     Qp, KVp = _pad128(Q), _pad128(KV)
-    m = dense_mask_on_device(fn, B, H, Qp, KVp, device)
+    m = dense_mask_on_device(fn, B, H, Qp, KVp, device, real=real or (Q, KV))
     name = getattr(fn, "__name__", "mask_mod")
     full_shape = torch.broadcast_shapes(m.shape, (1, 1, Qp, KVp))
     m = torch.broadcast_to(m, full_shape)

@@ -333,6 +333,20 @@ def test_affine_score_mod_tables(dev):
             run(dev, dtype, 2, 4, 2, 70, 150, 64, score=fn, oscore=fn, mask=causal_mask, omask=o_causal_mask,
                 strict=(dtype == torch.float16), opts=None if dtype == torch.float16 else {}, scale_maxabs=True)
 
+    # math_attention hands captured buffers to the mods as trailing arguments (attention.py:22-23)
+    def bias_from(score, b, h, q_idx, kv_idx, tab):
+        return score + tab[h.long(), (q_idx - kv_idx).clamp(-15, 15).long() + 15]
+
+    def doc_mask(b, h, q_idx, kv_idx, doc):
+        return doc[q_idx.long()] == doc[kv_idx.long()]
+    doc = torch.arange(96) // 20
+    q, k, v = seeded_qkv(1, 4, 4, 96, 96, 64, torch.float32)
+    out, lse2 = fa.math_attention(q.to(dev), k.to(dev), v.to(dev), bias_from, (doc_mask,), 0.125, {},
+                                  score_mod_other_buffers=(table_dev,), mask_mod_other_buffers=(doc.to(dev),))
+    want, want_lse = ref_attention(q, k, v, lambda s, b, h, qi, ki: bias_from(s, b, h, qi, ki, table),
+                                   lambda b, h, qi, ki: doc_mask(b, h, qi, ki, doc), scale=0.125, strict=True, return_lse=True)
+    assert max_abs(out.cpu(), want) <= 1e-4 and max_abs(lse2.cpu() * 0.6931471805599453, want_lse) <= 1e-4
+
     def quadratic(score, b, h, q_idx, kv_idx):
         return score * score
     q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 64, torch.float16))

@@ -255,3 +255,29 @@ def test_utils_score_matrix_and_picture(tmp_path):
     assert (tmp_path / "mask_picture.png").stat().st_size > 1000
     with pytest.raises(AssertionError):
         visualize_attention_scores(q, k)
+
+
+def test_mask_with_captured_buffer_is_not_indexed_past_the_end():
+    """The builder's padded index range (blockmask.py:440-444) must not reach a captured tensor: positions past
+    the real lengths are evaluated with clamped indices unless the mod provably computes from its index
+    arguments alone; such arithmetic mods still see them as if they were real."""
+    import functools
+    from flaxattention_amd.core.common import _index_arithmetic_only, dense_mask_on_device
+    from flaxattention_amd.masks import causal_mask, generate_sliding_window
+    table = torch.zeros(4)
+    assert _index_arithmetic_only(lambda b, h, q, kv: (q >= kv) & (q - kv < 7))
+    assert _index_arithmetic_only(causal_mask) and _index_arithmetic_only(generate_sliding_window(5))
+    assert _index_arithmetic_only(fa.and_masks(causal_mask, lambda b, h, q, kv: kv % 2 == 0))
+    assert not _index_arithmetic_only(lambda b, h, q, kv: table[q.long()] > 0)
+    assert not _index_arithmetic_only(functools.partial(lambda b, h, q, kv, t: t[q.long()] > 0, t=table))
+    assert not _index_arithmetic_only(fa.and_masks(causal_mask, lambda b, h, q, kv: table[kv.long()] > 0))
+    doc = torch.arange(96) // 20
+
+    def doc_mask(b, h, q_idx, kv_idx):
+        return doc[q_idx.long()] == doc[kv_idx.long()]
+    m = dense_mask_on_device(doc_mask, 1, 1, 128, 128, torch.device("cpu"), real=(96, 96))
+    assert m.shape == (1, 1, 128, 128)
+    qi, ki = torch.arange(128).clamp(max=95).view(128, 1), torch.arange(128).clamp(max=95).view(1, 128)
+    assert torch.equal(m[0, 0], doc[qi] == doc[ki])
+    causal = dense_mask_on_device(lambda b, h, q, kv: q >= kv, 1, 1, 128, 256, torch.device("cpu"), real=(100, 130))
+    assert torch.equal(causal[0, 0], torch.arange(128).view(128, 1) >= torch.arange(256).view(1, 256))
