@@ -124,27 +124,42 @@ def _identity(score, batch, head, token_q, token_kv):
 IDENTITY = ScoreMod(_lib.SCORE_IDENTITY, name="identity")
 
 
-def _probe_score_mod(fn: Callable, H: int) -> Optional[ScoreMod]:
+def _probe_score_mod(fn: Callable, H: int, shape: Optional[Tuple[int, int, int, int]] = None,
+                     device=None) -> Optional[ScoreMod]:
     """Recognise an untagged Python score_mod as one of the functor families by
-    evaluating it on a small CPU grid and checking every family exactly."""
-    P = 7
+    evaluating it on a small grid and checking every family exactly.  A callable that may look
+    positions up in captured tensors is only probed inside the real index ranges of `shape`
+    (an out-of-range index into a device tensor stops the process), and on the device when it
+    cannot take CPU tensors."""
+    Pq, Pkv, nb = 7, 9, 2
     Hn = max(int(H), 1)
-    s = torch.tensor([-1.75, -0.5, 0.0, 0.625, 2.5], dtype=torch.float32).reshape(5, 1, 1, 1, 1)
-    b = torch.arange(2, dtype=torch.int32).reshape(1, 2, 1, 1, 1)
-    h = torch.arange(Hn, dtype=torch.int32).reshape(1, 1, Hn, 1, 1)
-    q = torch.arange(P, dtype=torch.int32).reshape(1, 1, 1, P, 1)
-    kv = torch.arange(P + 2, dtype=torch.int32).reshape(1, 1, 1, 1, P + 2)
-    shape = (5, 2, Hn, P, P + 2)
-    try:
-        out = fn(s.expand(shape), b, h, q, kv)
-        if not torch.is_tensor(out):
+    if not _index_arithmetic_only(fn):
+        if shape is None:
             return None
-        out = torch.broadcast_to(out.to(torch.float32), shape)
-    except Exception:
+        nb, Pq, Pkv = min(nb, shape[0]), min(Pq, shape[2]), min(Pkv, shape[3])
+    s = torch.tensor([-1.75, -0.5, 0.0, 0.625, 2.5], dtype=torch.float32).reshape(5, 1, 1, 1, 1)
+    b = torch.arange(nb, dtype=torch.int32).reshape(1, nb, 1, 1, 1)
+    h = torch.arange(Hn, dtype=torch.int32).reshape(1, 1, Hn, 1, 1)
+    q = torch.arange(Pq, dtype=torch.int32).reshape(1, 1, 1, Pq, 1)
+    kv = torch.arange(Pkv, dtype=torch.int32).reshape(1, 1, 1, 1, Pkv)
+    shape5 = (5, nb, Hn, Pq, Pkv)
+    out = None
+    for where in ("cpu",) + ((device,) if device is not None else ()):
+        try:
+            res = fn(s.to(where).expand(shape5), b.to(where), h.to(where), q.to(where), kv.to(where))
+            if not torch.is_tensor(res):
+                return None
+            out = torch.broadcast_to(res.to(torch.float32), shape5).cpu()
+            s, b, h, q, kv = (t.to(where) for t in (s, b, h, q, kv))
+            break
+        except Exception:
+            continue
+    if out is None or Pkv < 2:
         return None
+    shape = shape5
 
     def same(c: ScoreMod) -> bool:
-        ref = torch.broadcast_to(_f32(c(s.expand(shape), b, h, q, kv)), shape)
+        ref = torch.broadcast_to(_f32(c(s.expand(shape), b, h, q, kv)), shape).cpu()
         return bool(torch.allclose(out, ref, rtol=1e-6, atol=1e-6))
 
     cands = [IDENTITY]
@@ -161,7 +176,7 @@ def _probe_score_mod(fn: Callable, H: int) -> Optional[ScoreMod]:
         cands.append(ScoreMod(_lib.SCORE_REL_BIAS, bias[0, 0, 0, 1].item(), name=getattr(fn, "__name__", "rel_bias")))
         # tanh soft-cap: cap from the saturated value
         try:
-            big = fn(torch.full((1, 1, 1, 1, 1), 1e9), b[:, :1], h[:, :, :1], q[..., :1, :], kv[..., :1])
+            big = fn(torch.full((1, 1, 1, 1, 1), 1e9, device=s.device), b[:, :1], h[:, :, :1], q[..., :1, :], kv[..., :1])
             cap = float(torch.as_tensor(big).reshape(-1)[0])
             if math.isfinite(cap) and cap > 0:
                 cands.append(ScoreMod(_lib.SCORE_TANH_SOFTCAP, cap, 1.0 / cap, name=getattr(fn, "__name__", "tanh_softcap")))
@@ -239,7 +254,7 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
     hit = _score_cache.get(key)
     if hit is not None and hit[0] is fn:
         return hit[1]
-    spec = _probe_score_mod(fn, H)
+    spec = _probe_score_mod(fn, H, shape, device)
     if spec is not None:
         _score_cache[key] = (fn, spec)
         return spec

@@ -197,6 +197,18 @@ def test_untagged_score_mod_is_recognised(dev):
         return score + (q_idx - kv_idx) * torch.exp2(-((h + 1) * 8.0 / 8))
     run(dev, torch.float32, 1, 8, 8, 64, 64, 32, score=my_alibi, oscore=o_alibi(8))
 
+    # the same bias with its slopes in a captured device tensor, for a single query row: the probe must stay
+    # inside the real index ranges and run on the device, and still find the ALiBi family (fused kernels)
+    from flaxattention_amd.core.common import resolve_score_mod
+    from flaxattention_amd import _lib
+    slopes = torch.exp2(-(torch.arange(8, device=dev) + 1.0))
+    per_row = torch.zeros(1, device=dev)      # one entry per query row: q_idx 1.. would be out of range
+
+    def slopes_alibi(score, b, h, q_idx, kv_idx):
+        return score + (q_idx - kv_idx) * slopes[h.long()] + per_row[q_idx.long()]
+    assert resolve_score_mod(slopes_alibi, 8, (2, 8, 1, 700), dev).kind == _lib.SCORE_ALIBI
+    run(dev, torch.float16, 2, 8, 8, 1, 700, 64, score=slopes_alibi, oscore=o_alibi(8), strict=False, grad=False)
+
     def unknown(score, b, h, q_idx, kv_idx):
         return score * score
     q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 32, torch.float32))
