@@ -21,6 +21,9 @@ selects numerics here:
                           whenever it applies (fp16/bf16, D = Dv in {64, 128},
                           at most 64 query rows per KV head, at least 512 keys)
     {"decode_splits": n}  force the split-KV decode kernel with n splits
+    {"pad_head_dim": bool}  16-bit inputs whose head sizes are not D = Dv in {64, 128} (but at most
+                          128) are zero-padded to the next of those so that the fused kernels serve
+                          them (default True)
 """
 from __future__ import annotations
 
@@ -277,6 +280,24 @@ def _as_kernel_layout(t: Array) -> Array:
     return t if t.stride(-1) == 1 else t.contiguous()
 
 
+def _pad_head_dims(q: Array, k: Array, v: Array, kernel_options) -> Tuple[Array, Array, Array]:
+    """The fused kernels exist for D = Dv in {64, 128}.  Other head sizes up to 128 (and Dv < D) of
+    16-bit inputs are zero-padded to the next of those: zero feature columns add nothing to Q.K^T, the
+    padded columns of O are dropped by the caller and the padded columns of the gradients are cut off by
+    autograd, so the result is the one of the original problem at matrix-core speed.  Opt out with
+    kernel_options={"pad_head_dim": False}; the faithful and the generic kernels take any size as it is."""
+    opts = kernel_options or {}
+    D, Dv = q.shape[-1], v.shape[-1]
+    if (q.dtype not in (torch.float16, torch.bfloat16) or opts.get("strict", False)
+            or opts.get("backend", "auto") == "generic" or not opts.get("pad_head_dim", True)):
+        return q, k, v
+    Dp = 64 if max(D, Dv) <= 64 else 128
+    if max(D, Dv) > 128 or (D == Dp and Dv == Dp):
+        return q, k, v
+    pad = torch.nn.functional.pad
+    return pad(q, (0, Dp - D)), pad(k, (0, Dp - D)), pad(v, (0, Dp - Dv))
+
+
 def math_attention(query: Array, key: Array, value: Array, score_mod: Callable, block_mask: Tuple, scale: float,
                    kernel_options: Dict[str, Any], score_mod_other_buffers: Tuple = (),
                    mask_mod_other_buffers: Tuple = (), use_pallas: bool = False) -> Tuple[Array, Array]:
@@ -330,9 +351,10 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
         block_mask = _create_empty_block_mask(query, key)
     if scale is None:
         scale = 1.0 / math.sqrt(query.shape[-1])
-    q, k, v = map(_as_kernel_layout, (query, key, value))
+    q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
     out, lse2 = _FlexAttention.apply(q, k, v, plan)
+    out = out[..., :value.shape[-1]]
     if return_lse:
         return out, lse2 * math.log(2.0)
     return out
@@ -378,7 +400,8 @@ def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Opt
         sm_scale = 1 / math.sqrt(query.shape[-1])
     if block_mask is not None and mask_mod is not None:
         raise ValueError("pass only one of block_mask= and mask_mod=")
-    q, k, v = map(_as_kernel_layout, (query, key, value))
+    q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
     out, _ = _FlexAttention.apply(q, k, v, plan)
+    out = out[..., :value.shape[-1]]
     return out if bhln else out.transpose(1, 2)

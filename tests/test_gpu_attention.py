@@ -270,6 +270,16 @@ def test_fused_bitmap_mask_dead_rows(dev):
     run(dev, torch.float16, 1, 2, 2, 768, 768, 64, mask=doc_mask, omask=doc_mask, strict=False)
 
 
+def test_fused_other_head_sizes_by_zero_padding(dev):
+    """D = 32, 96 and Dv < D reach the fused kernels through zero-padded feature columns."""
+    run(dev, torch.float16, 2, 4, 2, 130, 200, 32, mask=causal_mask, omask=o_causal_mask, strict=False, scale_maxabs=True)
+    run(dev, torch.bfloat16, 1, 4, 4, 100, 100, 96, score=generate_alibi_bias(4), oscore=o_alibi(4), strict=False, scale_maxabs=True)
+    run(dev, torch.float16, 1, 2, 2, 64, 300, 64, Dv=32, strict=False, scale_maxabs=True)
+    run(dev, torch.float16, 1, 2, 2, 64, 300, 80, Dv=48, strict=False, pallas=True, scale_maxabs=True)
+    # the generic kernels still take the sizes as they are
+    run(dev, torch.float16, 1, 2, 2, 40, 70, 32, strict=False, opts={"pad_head_dim": False}, scale_maxabs=True)
+
+
 def test_fused_fully_masked(dev):
     def fullmask(b, h, q_idx, kv_idx):
         return False
