@@ -307,9 +307,9 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   constexpr int DS = D / 16, DB = D / 32;
   // KV tiles land in LDS straight from global memory (global_load_lds, 16 bytes per lane, a wave
   // instruction fills 8 rows of 128 bytes), so rows are unpadded; the 16-byte chunk c of row r is
-  // kept at chunk position c ^ (r & 7), which makes both the row-fragment reads and the
+  // kept at chunk position c ^ lds_swz(r), which makes both the row-fragment reads and the
   // transposing reads conflict-free.  The lane that fills position (r, pos) therefore fetches
-  // chunk pos ^ (r & 7) of that row.
+  // chunk pos ^ lds_swz(r) of that row.
   constexpr int kTileElems = BN * D;  // 8 KB per tile
   __shared__ __align__(16) T Ksm[3][kTileElems];
   __shared__ __align__(16) T Vsm[3][kTileElems];
@@ -356,13 +356,13 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
   // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
-  const int fill_row = lane >> 3;                         // row inside the 8-row group = (row & 7)
-  const int fill_chunk = (lane & 7) ^ fill_row;           // logical chunk this lane fetches
+  const int fill_row = lane >> 3;                         // row inside the 8-row group
   auto issue_tile = [&](int stage, int kv0) {
     const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const int r0 = 16 * w + 8 * j;
+      const int fill_chunk = (lane & 7) ^ lds_swz<D>(8 * j + fill_row);  // logical chunk this lane fetches
       const int row = min(r0 + fill_row, lim);
       const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + fill_chunk * 8;
       const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + fill_chunk * 8;
@@ -376,29 +376,31 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   vec8 kfr[DS], vfr[2][DB], pf[2];
   int koff[DS];  // element offsets of this lane's K row fragments inside a 32-row block
 #pragma unroll
-  for (int s = 0; s < DS; s++) koff[s] = i32 * D + (((2 * s + g) ^ (i32 & 7)) * 8);
+  for (int s = 0; s < DS; s++) koff[s] = i32 * D + (((2 * s + g) ^ lds_swz<D>(i32)) * 8);
   auto read_k = [&](const T* Ks, int nb) {
 #pragma unroll
     for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(Ks + nb * 32 * D + koff[s]);
   };
-  // transposing reads: lane points at 4 elements of row 4g + (i16 >> 2) (+16tt, +8), logical column
+  // transposing reads: lane points at 4 elements of row 4g + (i16 >> 2) + 8e (+16tt), logical column
   // 32db + 16h + 4(i16 & 3)
-  int voff[DB];
+  int voff[2][DB];
   {
     const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
 #pragma unroll
-    for (int db = 0; db < DB; db++) {
-      const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
-      voff[db] = rl * D + ((chunk ^ (rl & 7)) * 8) + 4 * (i16 & 1);
-    }
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        voff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
+      }
   }
   auto read_v = [&](const T* Vs, int nb) {
 #pragma unroll
     for (int tt = 0; tt < 2; tt++)
 #pragma unroll
       for (int db = 0; db < DB; db++) {
-        const T* vp = Vs + (32 * nb + 16 * tt) * D + voff[db];
-        vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * D));
+        const T* vp = Vs + (32 * nb + 16 * tt) * D;
+        vfr[tt][db] = join8<vec8>(lds_read_tr(vp + voff[0][db]), lds_read_tr(vp + voff[1][db]));
       }
   };
 
