@@ -371,11 +371,13 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 }
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
-  // aim for one resident generation of workgroups on 256 CUs: three per CU with up to 32 query
-  // columns (three waves per SIMD), two per CU with 64; at least 8 steps each
+  // aim for one resident generation of workgroups on 256 CUs, as many per CU as the kernel's
+  // registers allow: D = 64: three with up to 32 query columns, two with 64; D = 128: two and one;
+  // at least 8 steps each
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
-  const int slots = (p.Hq / p.Hkv) * p.Lq > 32 ? 512 : 768;
+  const bool wide = (p.Hq / p.Hkv) * p.Lq > 32;
+  const int slots = p.D == 64 ? (wide ? 512 : 768) : (wide ? 256 : 512);
   int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
