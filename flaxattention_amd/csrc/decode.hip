@@ -10,7 +10,9 @@
 // Per step and wave:
 //   K rows go straight from global memory into MFMA A-operand registers
 //   (lane i holds 16-byte pieces of row kv0 + i%32) -- no LDS round trip;
-//   V rows pass through a wave-private LDS strip to be read back transposed.
+//   V rows are fetched global -> LDS directly into one of two wave-private strips
+//   (unpadded, swizzled) and read back transposed; with more than 32 columns the Q
+//   fragments are re-read from LDS every step, which keeps three waves per SIMD at D = 64.
 //   All query heads that share a KV head (GQA) are packed into the N columns of
 //   the MFMA, so K and V are read once per group.
 // Each workgroup writes an unnormalised partial (O, m, l) per column; a second
@@ -22,15 +24,23 @@ namespace flex {
 constexpr int kStep = 32;  // KV rows per wave step
 
 template <typename T, int D, int KIND, bool ROUND_S, int NB>
-__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 3 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits) {
   typedef typename Frag<T>::vec8 vec8;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NV = kStep * CPR / 64;
-  __shared__ __align__(16) T Vs[4][kStep * ROWE];
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8;
+  constexpr int RPI = 64 / CPR;        // V rows one wave-wide fetch instruction fills
+  constexpr int NVI = kStep / RPI;     // fetch instructions per step
+  // V strips: per wave two stages of 32 unpadded swizzled rows, filled global -> LDS directly (no staging
+  // registers).  The same memory serves the cross-wave reduction of the partial outputs at the end.
+  constexpr int kStripElems = kStep * D;
+  constexpr int kVsBytes = 4 * 2 * kStripElems * (int)sizeof(T), kRedBytes = 4 * 16 * 64 * (int)sizeof(float);
+  __shared__ __align__(16) unsigned char vs_red[kVsBytes > kRedBytes ? kVsBytes : kRedBytes];
   __shared__ float mbuf[4][NB][32];
-  __shared__ __align__(16) float red[4][16][64];
+  // with two column blocks the Q fragments are re-read from LDS every step instead of living in registers
+  __shared__ __align__(16) T Qs[NB == 2 ? 64 * ROWE : 8];
+  float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(vs_red);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave index, provably uniform: step addresses stay scalar
@@ -53,7 +63,12 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     const T* qp = q + b * p.q_stride[0] + col_h[nb] * p.q_stride[1] + (int64_t)col_q[nb] * p.q_stride[2] + 8 * g;
 #pragma unroll
     for (int s = 0; s < DS; s++) qf[nb][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+    if (NB == 2 && w == 0) {
+#pragma unroll
+      for (int s = 0; s < DS; s++) *reinterpret_cast<vec8*>(Qs + (nb * 32 + i32) * ROWE + 16 * s + 8 * g) = qf[nb][s];
+    }
   }
+  if (NB == 2) __syncthreads();
 
   // schedule: list entries (64-row tiles of query block 0) when given and G == 1, else every step
   const FlexTileLists& tl = p.tiles;
@@ -89,20 +104,36 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   // it is finite.
   const int last = p.Lkv - 1;
   vec8 kfr[DS];
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  u32x4 vreg[NV];
-  auto load_step = [&](int kv0) {
+  T* Vw = reinterpret_cast<T*>(vs_red) + w * 2 * kStripElems;
+  const int fill_row = lane / CPR, fill_pos = lane % CPR;
+  // V first, K last: loads return in order, so once the K registers of a step have arrived (the
+  // compiler waits for them before the first MFMA) the V strip of that step has landed too
+  auto load_step = [&](int kv0, int stage) {
     const int lim = last - kv0;  // last valid row of this step, relative
+    const T* vp = vbase + (int64_t)kv0 * vs2;
+#pragma unroll
+    for (int j = 0; j < NVI; j++) {
+      const int r = RPI * j + fill_row;
+      const T* vg = vp + min(r, lim) * (int)vs2 + ((fill_pos ^ lds_swz<D>(r)) * 8);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                       (__attribute__((address_space(3))) void*)(Vw + stage * kStripElems + RPI * j * D), 16, 0, 0);
+    }
     const T* kp = kbase + (int64_t)kv0 * ks2 + min(i32, lim) * (int)ks2 + 8 * g;
 #pragma unroll
     for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
-    const T* vp = vbase + (int64_t)kv0 * vs2;
-#pragma unroll
-    for (int j = 0; j < NV; j++) {
-      const int c = lane + 64 * j, r = c / CPR, cc = c % CPR;
-      vreg[j] = *reinterpret_cast<const u32x4*>(vp + min(r, lim) * (int)vs2 + cc * 8);
-    }
   };
+  // transposing reads of a strip: 4 elements of row 4g + (i16 >> 2) + 8e (+16t), logical column 32db + 16hh + 4(i16 & 3)
+  int voff[2][DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
+#pragma unroll
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        voff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
+      }
+  }
 
   Score2<KIND> sm[NB];
   float m_run[NB], l_run[NB];
@@ -118,7 +149,6 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
       for (int r = 0; r < 16; r++) oacc[nb][db][r] = 0.f;
   }
   const bool trivial_mask = p.mask.kind == FLEX_MASK_BAND && p.mask.lo == INT32_MIN && p.mask.hi == INT32_MAX;
-  T* Vw = Vs[w];
   constexpr float kTau = 8.f;
 
   // KV offsets are looked up two visits ahead so that the (dependent) tile-index
@@ -127,8 +157,9 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   int kv_cur = st < st_end ? step_kv0(st) : 0;
   int kv_nx1 = st + 4 < st_end ? step_kv0(st + 4) : 0;
   int kv_nx2 = st + 8 < st_end ? step_kv0(st + 8) : 0;
-  if (st < st_end) load_step(kv_cur);
-  for (; st < st_end; st += 4) {
+  int stage = 0;
+  if (st < st_end) load_step(kv_cur, 0);
+  for (; st < st_end; st += 4, stage ^= 1) {
     const int kv0 = kv_cur;
     // scores first: they consume the K registers, which the next step's loads then reuse
     float16_t s_a, s_b;  // named (not an array) so that they stay in registers
@@ -136,15 +167,16 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     for (int r = 0; r < 16; r++) { s_a[r] = 0.f; s_b[r] = 0.f; }
 #pragma unroll
     for (int s = 0; s < DS; s++) {
-      s_a = Frag<T>::mfma(kfr[s], qf[0][s], s_a);
-      if (NB > 1) s_b = Frag<T>::mfma(kfr[s], qf[NB - 1][s], s_b);
+      if (NB == 1) {
+        s_a = Frag<T>::mfma(kfr[s], qf[0][s], s_a);
+      } else {
+        const T* qp = Qs + i32 * ROWE + 16 * s + 8 * g;
+        s_a = Frag<T>::mfma(kfr[s], *reinterpret_cast<const vec8*>(qp), s_a);
+        s_b = Frag<T>::mfma(kfr[s], *reinterpret_cast<const vec8*>(qp + 32 * ROWE), s_b);
+      }
     }
-#pragma unroll
-    for (int j = 0; j < NV; j++) {
-      const int c = lane + 64 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<u32x4*>(Vw + r * ROWE + cc * 8) = vreg[j];
-    }
-    if (st + 4 < st_end) load_step(kv_nx1);
+    // this step's V strip landed with its K registers; the other strip was last read a step ago
+    if (st + 4 < st_end) load_step(kv_nx1, stage ^ 1);
     kv_cur = kv_nx1;
     kv_nx1 = kv_nx2;
     if (st + 12 < st_end) kv_nx2 = step_kv0(st + 12);
@@ -201,15 +233,14 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
         pf[nb][tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
       }
     }
-    // the V strip was written by this wave only and LDS operations of one wave
-    // complete in order: no workgroup barrier is needed before reading it back
+    // the V strips belong to this wave alone: no workgroup barrier is needed
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int t = 0; t < 2; t++) {
 #pragma unroll
       for (int db = 0; db < DB; db++) {
-        const T* vp = Vw + (16 * t + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-        vec8 a = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+        const T* vp = Vw + stage * kStripElems + 16 * t * D;
+        vec8 a = join8<vec8>(lds_read_tr(vp + voff[0][db]), lds_read_tr(vp + voff[1][db]));
 #pragma unroll
         for (int nb = 0; nb < NB; nb++) oacc[nb][db] = Frag<T>::mfma(a, pf[nb][t], oacc[nb][db]);
       }
@@ -372,12 +403,12 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
   // aim for one resident generation of workgroups on 256 CUs, as many per CU as the kernel's
-  // registers allow: D = 64: three with up to 32 query columns, two with 64; D = 128: two and one;
+  // registers allow: D = 64: three; D = 128: two with up to 32 query columns, one with 64;
   // at least 8 steps each
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
   const bool wide = (p.Hq / p.Hkv) * p.Lq > 32;
-  const int slots = p.D == 64 ? (wide ? 512 : 768) : (wide ? 256 : 512);
+  const int slots = p.D == 64 ? 768 : (wide ? 256 : 512);
   int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
