@@ -134,7 +134,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   }
 
   Score2<KIND> sm;
-  sm.init(p.score, p.scale, h);
+  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
   Mask2 visible(p.mask, b, h, p.Lkv);
   float16_t dqacc[DB];
 #pragma unroll
@@ -313,7 +313,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 
   for (int gi = 0; gi < G; gi++) {
     const int h = hk * G + gi;
-    sm.init(p.score, p.scale, h);
+    sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
     Mask2 visible(p.mask, b, h, p.Lkv);
     const int32_t* full_idx = nullptr;
     const int32_t* part_idx = nullptr;
@@ -572,6 +572,7 @@ static int launch_kind(const FlexAttnParams& p, const void* q, const void* k, co
     case FLEX_SCORE_ALIBI: return launch_rs<T, D, FLEX_SCORE_ALIBI>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
     case FLEX_SCORE_TANH_SOFTCAP: return launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
     case FLEX_SCORE_REL_BIAS: return launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+    case FLEX_SCORE_AFFINE: return launch_rs<T, D, FLEX_SCORE_AFFINE>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
   }
   return 1;
 }

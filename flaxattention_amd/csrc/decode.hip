@@ -397,7 +397,7 @@ void flex_set_error(const char* fmt, ...);
 bool flex_mfma_shape_ok(const FlexAttnParams& p);
 
 bool flex_decode_supported(const FlexAttnParams& p) {
-  if (!flex_mfma_shape_ok(p)) return false;
+  if (!flex_mfma_shape_ok(p) || p.score.kind == FLEX_SCORE_AFFINE) return false;
   return (int64_t)(p.Hq / p.Hkv) * p.Lq <= 64 && p.Hkv <= 65535 && p.B <= 65535;
 }
 

@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   };
 
   Score2<KIND> sm;
-  sm.init(p.score, p.scale, h);
+  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
   Mask2 visible(p.mask, b, h, p.Lkv);
 
   float16_t oacc[RQ][DB];
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   };
 
   Score2<KIND> sm;
-  sm.init(p.score, p.scale, h);
+  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
   Mask2 visible(p.mask, b, h, p.Lkv);
 
   float16_t oacc[RQ][DB], s_cur;
@@ -595,13 +595,16 @@ static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, con
   // D = 64 without tile lists (every workgroup has the same work): the pipelined kernel with
   // 256-row workgroups.  With lists the 128-row kernel: twice the workgroups, half the length of the
   // longest one, which is what bounds a causal-like schedule.
-  if (D == 64 && !p.tiles.kv_num) {
-    dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
-    if (p.flags & FLEX_ROUND_S)
-      hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
-    else
-      hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
-    return;
+  // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
+  if constexpr (KIND != FLEX_SCORE_AFFINE) {
+    if (D == 64 && !p.tiles.kv_num) {
+      dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
+      if (p.flags & FLEX_ROUND_S)
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+      else
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+      return;
+    }
   }
   dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B);
   if (p.flags & FLEX_ROUND_S)
@@ -618,6 +621,7 @@ static int launch_kind(const FlexAttnParams& p, const void* q, const void* k, co
     case FLEX_SCORE_ALIBI: launch_rs<T, D, FLEX_SCORE_ALIBI>(p, q, k, v, o, lse2, s); return 0;
     case FLEX_SCORE_TANH_SOFTCAP: launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, q, k, v, o, lse2, s); return 0;
     case FLEX_SCORE_REL_BIAS: launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, q, k, v, o, lse2, s); return 0;
+    case FLEX_SCORE_AFFINE: launch_rs<T, D, FLEX_SCORE_AFFINE>(p, q, k, v, o, lse2, s); return 0;
   }
   return 1;
 }
@@ -632,7 +636,8 @@ static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0
 // dtype / head size / layout the MFMA kernels can take at all
 bool flex_mfma_shape_ok(const FlexAttnParams& p) {
   if (p.dtype != FLEX_F16 && p.dtype != FLEX_BF16) return false;
-  if (p.score.kind == FLEX_SCORE_AFFINE) return false;  // dense tables: generic kernels only
+  // dense tables: an additive one is fused (read per block); a multiplicative one goes to the generic kernels
+  if (p.score.kind == FLEX_SCORE_AFFINE && (p.score.mul || !p.score.add)) return false;
   if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
   if (!strides_ok(p.q_stride) || !strides_ok(p.k_stride) || !strides_ok(p.v_stride) || !strides_ok(p.o_stride)) return false;
   if ((int64_t)((p.Lq + 127) / 128) * p.Hq * p.B > 0x7fffffff) return false;

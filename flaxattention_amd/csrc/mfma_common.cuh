@@ -76,7 +76,7 @@ template <int KIND> struct Score2;
 template <> struct Score2<FLEX_SCORE_IDENTITY> {
   static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c;
-  __device__ __forceinline__ void init(const FlexScoreMod&, float scale, int h) { c = scale * kLog2e; }
+  __device__ __forceinline__ void init(const FlexScoreMod&, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) { c = scale * kLog2e; }
   __device__ __forceinline__ void tile(int q, int kvb) {}
   __device__ __forceinline__ void tileT(int qb, int kv) {}
   __device__ __forceinline__ float apply(float s, int off) const { return s * c; }
@@ -89,7 +89,7 @@ template <> struct Score2<FLEX_SCORE_CHECKERBOARD> {
   float c0, c1, f0, f1;  // factor (x scale x log2e) for even / odd parity
   float ce, co, fe, fo;  // the same, resolved for even / odd `off` of this lane
   int by_kv;
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     f0 = m.p0; f1 = m.p1; c0 = m.p0 * scale * kLog2e; c1 = m.p1 * scale * kLog2e; by_kv = m.i0;
   }
   __device__ __forceinline__ void tile(int q, int kvb) {
@@ -115,7 +115,7 @@ constexpr int kScoreCheckerboardKv = 100;
 template <> struct Score2<kScoreCheckerboardKv> {
   static constexpr bool kGradOne = true;  // inside the loop; see key_grad
   float c0, c1, f0, f1, ck, key_grad;
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     f0 = m.p0; f1 = m.p1; c0 = m.p0 * scale * kLog2e; c1 = m.p1 * scale * kLog2e;
   }
   __device__ __forceinline__ void tileT(int qb, int kv) {
@@ -135,7 +135,7 @@ template <> struct Score2<kScoreCheckerboardFold> {
   float c0, c1, l0, l1;
   float ce, co, le, lo;
   int by_kv;
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     c0 = m.p0 * scale * kLog2e; c1 = m.p1 * scale * kLog2e; l0 = log2f(m.p0); l1 = log2f(m.p1); by_kv = m.i0;
   }
   __device__ __forceinline__ void tile(int q, int kvb) {
@@ -152,7 +152,7 @@ template <> struct Score2<kScoreCheckerboardFold> {
 template <> struct Score2<FLEX_SCORE_ALIBI> {
   static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     c = scale * kLog2e;
     slope2 = m.p0 * exp2f(-((float)(h + 1) * 8.0f / (float)m.i0)) * kLog2e;
   }
@@ -166,7 +166,7 @@ template <> struct Score2<FLEX_SCORE_ALIBI> {
 template <> struct Score2<FLEX_SCORE_REL_BIAS> {
   static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
   float c, slope2, base, step;
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     c = scale * kLog2e;
     slope2 = m.p0 * kLog2e;
   }
@@ -180,7 +180,7 @@ template <> struct Score2<FLEX_SCORE_REL_BIAS> {
 template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
   static constexpr bool kGradOne = false;  // d score_mod / d score == 1 everywhere
   float a, cap2, sc;  // a = 2*log2e*scale/cap, cap2 = cap*log2e
-  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h) {
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
     a = 2.f * kLog2e * scale * m.p1; cap2 = m.p0 * kLog2e; sc = scale;
   }
   __device__ __forceinline__ void tile(int q, int kvb) {}
@@ -192,6 +192,40 @@ template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
   __device__ __forceinline__ float apply(float s, int off) const { return cap2 * tanh_(s); }
   __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(cap2, tanh_(s), -m); }
   __device__ __forceinline__ float grad(float s, int off) const { float t = tanh_(s); return 1.f - t * t; }
+};
+
+// score + add[b,h,q,kv] from a dense fp32 table (FLEX_SCORE_AFFINE without a multiplicative table:
+// what a score_mod that adds a captured bias is lowered to).  The 16 table entries of a lane's
+// block are fetched when the block is entered; indices are clamped to the table (entries past the
+// ends of the sequences are masked out by the caller whatever they hold).
+template <> struct Score2<FLEX_SCORE_AFFINE> {
+  static constexpr bool kGradOne = true;  // d score_mod / d score == 1 everywhere
+  float c;
+  const float* add_bh;
+  int64_t sq;
+  int q_last, kv_last;
+  float bias[16];  // log2(e) * add for accumulator register r (key / query offset acc_row(r))
+  static __device__ __forceinline__ constexpr int reg_of(int off) { return 4 * (off / 8) + (off % 4); }
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
+    c = scale * kLog2e;
+    add_bh = m.add + b * m.stride_b + h * m.stride_h;
+    sq = m.stride_q;
+    q_last = Lq - 1;
+    kv_last = Lkv - 1;
+  }
+  __device__ __forceinline__ void tile(int q, int kvb) {
+    const float* row = add_bh + (int64_t)min(q, q_last) * sq;
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias[r] = row[min(kvb + acc_row(r), kv_last)] * kLog2e;
+  }
+  __device__ __forceinline__ void tileT(int qb, int kv) {
+    const float* col = add_bh + min(kv, kv_last);
+#pragma unroll
+    for (int r = 0; r < 16; r++) bias[r] = col[(int64_t)min(qb + acc_row(r), q_last) * sq] * kLog2e;
+  }
+  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s, c, bias[reg_of(off)]); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(s, c, bias[reg_of(off)] - m); }
+  __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
 // band / bitmap mask evaluated at (q, kv)

@@ -39,8 +39,9 @@ enum FlexScoreKind {
   FLEX_SCORE_AFFINE = 5        /* mul[b,h,q,kv] * score + add[b,h,q,kv] from dense fp32
                                   tables: what a Python score_mod that is affine in the score
                                   (captured bias tables, position-dependent scaling;
-                                  attention.py:22-23, 59-63) is lowered to.  Served by the
-                                  generic kernels only. */
+                                  attention.py:22-23, 59-63) is lowered to.  An additive
+                                  table alone (mul == NULL) is read by the fused kernels;
+                                  with a multiplicative table the generic kernels serve it. */
 };
 
 typedef struct FlexScoreMod {

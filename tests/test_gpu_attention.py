@@ -337,6 +337,35 @@ def test_fused_seeded_sweep(dev, seed):
             mask=c["mask"], omask=c["omask"], strict=False, scale_maxabs=True)
 
 
+# ---- score_mods that add a captured bias: a dense additive table read by the fused kernels ----
+def test_fused_additive_bias_table(dev):
+    g = torch.Generator().manual_seed(11)
+    rel = torch.randn(6, 63, generator=g)            # per-head relative-position bias (T5 style)
+    full = torch.randn(2, 1, 150, 333, generator=g)  # a bias given per (batch, query, key), shared by the heads
+    rel_dev, full_dev = rel.to(dev), full.to(dev)
+
+    def rel_bias(score, b, h, q_idx, kv_idx):
+        t = rel_dev if score.is_cuda else rel
+        return score + t[h.long(), (kv_idx - q_idx).clamp(-31, 31).long() + 31]
+
+    def full_bias(score, b, h, q_idx, kv_idx):
+        t = full_dev if score.is_cuda else full
+        return score + t[b.long(), 0, q_idx.long(), kv_idx.long()]
+    from flaxattention_amd.core.common import resolve_score_mod
+    from flaxattention_amd import _lib
+    spec = resolve_score_mod(rel_bias, 6, (2, 6, 200, 200), dev)
+    assert spec.kind == _lib.SCORE_AFFINE and spec.mul is None and spec.add.shape == (1, 6, 200, 200)
+    for dtype, D in ((torch.float16, 64), (torch.bfloat16, 128)):
+        print(f"case additive table rel_bias {dtype} D{D}", flush=True)
+        run(dev, dtype, 2, 6, 6, 200, 200, D, score=rel_bias, oscore=rel_bias, mask=causal_mask, omask=o_causal_mask,
+            strict=False, scale_maxabs=True)
+        run(dev, dtype, 2, 6, 2, 130, 257, D, score=rel_bias, oscore=rel_bias, strict=False, scale_maxabs=True)   # GQA, ragged
+    print("case additive table full_bias", flush=True)
+    run(dev, torch.float16, 2, 4, 4, 150, 333, 64, score=full_bias, oscore=full_bias, mask=generate_sliding_window(40),
+        omask=o_sliding_window(40), strict=False, scale_maxabs=True)
+    run(dev, torch.float16, 2, 4, 4, 150, 333, 64, score=full_bias, oscore=full_bias, strict=False, pallas=True, scale_maxabs=True)
+
+
 # ---- score_mods outside the functor families: lowered to dense affine tables, generic kernels ----
 def test_affine_score_mod_tables(dev):
     table = torch.randn(4, 31, generator=torch.Generator().manual_seed(7))
