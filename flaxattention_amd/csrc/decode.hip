@@ -11,8 +11,8 @@
 //   K rows go straight from global memory into MFMA A-operand registers
 //   (lane i holds 16-byte pieces of row kv0 + i%32) -- no LDS round trip;
 //   V rows are fetched global -> LDS directly into one of two wave-private strips
-//   (unpadded, swizzled) and read back transposed; with more than 32 columns the Q
-//   fragments are re-read from LDS every step, which keeps three waves per SIMD at D = 64.
+//   (unpadded, swizzled) and read back transposed; with more than 32 columns at D = 128
+//   the Q fragments are re-read from LDS every step.
 //   All query heads that share a KV head (GQA) are packed into the N columns of
 //   the MFMA, so K and V are read once per group.
 // Each workgroup writes an unnormalised partial (O, m, l) per column; a second
@@ -24,7 +24,7 @@ namespace flex {
 constexpr int kStep = 32;  // KV rows per wave step
 
 template <typename T, int D, int KIND, bool ROUND_S, int NB>
-__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 3 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits) {
@@ -38,8 +38,9 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 3 : 1
   constexpr int kVsBytes = 4 * 2 * kStripElems * (int)sizeof(T), kRedBytes = 4 * 16 * 64 * (int)sizeof(float);
   __shared__ __align__(16) unsigned char vs_red[kVsBytes > kRedBytes ? kVsBytes : kRedBytes];
   __shared__ float mbuf[4][NB][32];
-  // with two column blocks the Q fragments are re-read from LDS every step instead of living in registers
-  __shared__ __align__(16) T Qs[NB == 2 ? 64 * ROWE : 8];
+  // two column blocks at D = 128: the Q fragments (64 registers) are re-read from LDS every step instead
+  constexpr bool kQInLds = NB == 2 && D == 128;
+  __shared__ __align__(16) T Qs[kQInLds ? 64 * ROWE : 8];
   float (*red)[16][64] = reinterpret_cast<float (*)[16][64]>(vs_red);
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -63,12 +64,12 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 3 : 1
     const T* qp = q + b * p.q_stride[0] + col_h[nb] * p.q_stride[1] + (int64_t)col_q[nb] * p.q_stride[2] + 8 * g;
 #pragma unroll
     for (int s = 0; s < DS; s++) qf[nb][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
-    if (NB == 2 && w == 0) {
+    if (kQInLds && w == 0) {
 #pragma unroll
       for (int s = 0; s < DS; s++) *reinterpret_cast<vec8*>(Qs + (nb * 32 + i32) * ROWE + 16 * s + 8 * g) = qf[nb][s];
     }
   }
-  if (NB == 2) __syncthreads();
+  if (kQInLds) __syncthreads();
 
   // schedule: list entries (64-row tiles of query block 0) when given and G == 1, else every step
   const FlexTileLists& tl = p.tiles;
@@ -167,8 +168,9 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 3 : 1
     for (int r = 0; r < 16; r++) { s_a[r] = 0.f; s_b[r] = 0.f; }
 #pragma unroll
     for (int s = 0; s < DS; s++) {
-      if (NB == 1) {
+      if (!kQInLds) {
         s_a = Frag<T>::mfma(kfr[s], qf[0][s], s_a);
+        if (NB > 1) s_b = Frag<T>::mfma(kfr[s], qf[NB - 1][s], s_b);
       } else {
         const T* qp = Qs + i32 * ROWE + 16 * s + 8 * g;
         s_a = Frag<T>::mfma(kfr[s], *reinterpret_cast<const vec8*>(qp), s_a);
@@ -403,12 +405,12 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
   // aim for one resident generation of workgroups on 256 CUs, as many per CU as the kernel's
-  // registers allow: D = 64: three; D = 128: two with up to 32 query columns, one with 64;
+  // registers allow: D = 64: three with up to 32 query columns, two with 64; D = 128: two and one;
   // at least 8 steps each
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
   const bool wide = (p.Hq / p.Hkv) * p.Lq > 32;
-  const int slots = p.D == 64 ? 768 : (wide ? 256 : 512);
+  const int slots = p.D == 64 ? (wide ? 512 : 768) : (wide ? 256 : 512);
   int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
