@@ -250,24 +250,29 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
         return IDENTITY
     if isinstance(fn, ScoreMod):
         return fn
+    # a lowering is cached only together with what it was derived from: the callable and the captured tensors
+    # at their current versions (a learned bias that the optimizer has updated in place must be read again)
+    stamp = _capture_stamp(fn)
     key = (id(fn), H)
     hit = _score_cache.get(key)
-    if hit is not None and hit[0] is fn:
+    if hit is not None and hit[0] is fn and _stamp_valid(hit[2]):
         return hit[1]
     spec = _probe_score_mod(fn, H, shape, device)
     if spec is not None:
-        _score_cache[key] = (fn, spec)
+        if stamp is not None:
+            _score_cache[key] = (fn, spec, stamp)
         return spec
     if shape is not None and device is not None:
         key = (id(fn),) + tuple(shape) + (str(device),)
         hit = _score_cache.get(key)
-        if hit is not None and hit[0] is fn:
+        if hit is not None and hit[0] is fn and _stamp_valid(hit[2]):
             return hit[1]
         spec = affine_score_mod(fn, *shape, device)
         if spec is not None:
             if len(_score_cache) > 64:
                 _score_cache.clear()
-            _score_cache[key] = (fn, spec)
+            if stamp is not None:
+                _score_cache[key] = (fn, spec, stamp)
             return spec
     raise NotImplementedError(
         "score_mod is neither one of the fused functor families (identity, checkerboard, ALiBi, tanh soft-cap, "
@@ -382,32 +387,41 @@ def _eval_mask(fn: Callable, b, h, q, kv) -> torch.Tensor:
     return m.to(torch.bool)
 
 
-def _index_arithmetic_only(fn, depth: int = 0) -> bool:
-    """True when `fn` provably computes from its index arguments alone: everything it closes over, defaults to
-    or reads from its globals is a number, a string, a module or another such function.  Anything else (a
-    tensor, an array, an object that may hold one) makes it a mod that may look positions up in a buffer."""
+def _scan_captures(fn, tensors: list, depth: int = 0) -> bool:
+    """Walk what `fn` closes over, defaults to or reads from its globals.  Tensors found on the way are
+    appended to `tensors`; the return value says whether everything else was transparent: numbers, strings,
+    modules, containers of such, and functions that are themselves transparent.  An object of any other kind
+    (an array, a module instance, a bound method) may hold state this walk cannot see."""
     import functools
     import types
 
     def plain(x) -> bool:
         if x is None or isinstance(x, (bool, int, float, complex, str, bytes, types.ModuleType, type)):
             return True
+        if torch.is_tensor(x):
+            tensors.append(x)
+            return True
         if isinstance(x, MaskMod):
-            return x.bits is None
+            if x.bits is not None:
+                tensors.append(x.bits)
+            return True
+        if isinstance(x, ScoreMod):
+            tensors.extend(t for t in (x.mul, x.add) if t is not None)
+            return True
         if isinstance(x, (tuple, list, frozenset, set)):
-            return all(plain(y) for y in x)
+            return all([plain(y) for y in x])
         if isinstance(x, dict):
-            return all(plain(y) for y in x.values())
+            return all([plain(y) for y in x.values()])
         if isinstance(x, (types.FunctionType, types.BuiltinFunctionType, functools.partial)):
-            return _index_arithmetic_only(x, depth + 1)
+            return _scan_captures(x, tensors, depth + 1)
         return False
 
     if depth > 4:
         return False
-    if isinstance(fn, MaskMod):
-        return fn.bits is None
+    if isinstance(fn, (MaskMod, ScoreMod)):
+        return plain(fn)
     if isinstance(fn, functools.partial):
-        return plain(fn.func) and plain(fn.args) and plain(fn.keywords)
+        return all([plain(fn.func), plain(fn.args), plain(fn.keywords)])
     if isinstance(fn, types.BuiltinFunctionType):
         return True
     code = getattr(fn, "__code__", None)
@@ -416,7 +430,28 @@ def _index_arithmetic_only(fn, depth: int = 0) -> bool:
     seen = [c.cell_contents for c in (fn.__closure__ or ())]
     seen += list(fn.__defaults__ or ()) + list((fn.__kwdefaults__ or {}).values())
     seen += [fn.__globals__[n] for n in code.co_names if n in fn.__globals__]
-    return all(plain(x) for x in seen)
+    return all([plain(x) for x in seen])
+
+
+def _index_arithmetic_only(fn) -> bool:
+    """True when `fn` provably computes from its index arguments alone: everything it closes over, defaults to
+    or reads from its globals is a number, a string, a module or another such function.  Anything else (a
+    tensor, an array, an object that may hold one) makes it a mod that may look positions up in a buffer."""
+    tensors: list = []
+    return _scan_captures(fn, tensors) and not tensors
+
+
+def _capture_stamp(fn):
+    """What a cached lowering of `fn` depends on besides `fn` itself: the captured tensors with their version
+    counters, or None when `fn` holds state that cannot be seen (then nothing about it may be cached)."""
+    tensors: list = []
+    if not _scan_captures(fn, tensors):
+        return None
+    return [(t, t._version) for t in tensors]
+
+
+def _stamp_valid(stamp) -> bool:
+    return all(t._version == v for t, v in stamp)
 
 
 def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device,

@@ -360,6 +360,15 @@ def test_fused_additive_bias_table(dev):
         run(dev, dtype, 2, 6, 6, 200, 200, D, score=rel_bias, oscore=rel_bias, mask=causal_mask, omask=o_causal_mask,
             strict=False, scale_maxabs=True)
         run(dev, dtype, 2, 6, 2, 130, 257, D, score=rel_bias, oscore=rel_bias, strict=False, scale_maxabs=True)   # GQA, ragged
+    # the table is a snapshot of the captured tensor: an in-place update (a learned bias after an optimizer step)
+    # must be seen by the next call
+    q, k, v = seeded_qkv(1, 6, 6, 64, 64, 64, torch.float16)
+    before = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=rel_bias)
+    rel_dev.mul_(-3.0)
+    rel.mul_(-3.0)
+    after = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=rel_bias)
+    want = ref_attention(q, k, v, rel_bias, None, strict=True)
+    assert rel_l2(after.cpu(), want) <= 1e-3 and rel_l2(before.cpu(), want) > 1e-1
     print("case additive table full_bias", flush=True)
     run(dev, torch.float16, 2, 4, 4, 150, 333, 64, score=full_bias, oscore=full_bias, mask=generate_sliding_window(40),
         omask=o_sliding_window(40), strict=False, scale_maxabs=True)

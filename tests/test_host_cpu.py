@@ -281,3 +281,20 @@ def test_mask_with_captured_buffer_is_not_indexed_past_the_end():
     assert torch.equal(m[0, 0], doc[qi] == doc[ki])
     causal = dense_mask_on_device(lambda b, h, q, kv: q >= kv, 1, 1, 128, 256, torch.device("cpu"), real=(100, 130))
     assert torch.equal(causal[0, 0], torch.arange(128).view(128, 1) >= torch.arange(256).view(1, 256))
+
+
+def test_cached_lowerings_follow_captured_tensors():
+    """A lowering of a score_mod is reused only while the tensors the callable captures are unchanged."""
+    from flaxattention_amd.core.common import _capture_stamp, _stamp_valid
+    table = torch.zeros(4)
+    fn = lambda s, b, h, q, kv: s + table[h.long()]   # noqa: E731
+    stamp = _capture_stamp(fn)
+    assert stamp is not None and len(stamp) == 1 and stamp[0][0] is table and _stamp_valid(stamp)
+    table.add_(1.0)
+    assert not _stamp_valid(stamp)
+    assert _capture_stamp(lambda s, b, h, q, kv: s * 2.0) == []
+
+    class Holder:
+        t = torch.ones(2)
+    holder = Holder()
+    assert _capture_stamp(lambda s, b, h, q, kv: s + holder.t[0]) is None   # state that cannot be seen: never cached
