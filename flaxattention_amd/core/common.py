@@ -73,13 +73,20 @@ class ScoreMod:
         self.kind, self.p0, self.p1, self.i0 = int(kind), float(p0), float(p1), int(i0)
         self.__name__ = name
         # SCORE_AFFINE: dense fp32 tables [b', h', q', Lkv] (each leading extent 1 or full) and the
-        # callable they were read from
+        # callable they were read from.  An additive table whose diagonals are constant (a bias that depends
+        # on kv_idx - q_idx only) is kept as [b', h', Lq + Lkv - 1] instead, entry (kv - q) + diag_zero: the
+        # kernels' address  add + q * stride_q + kv  reaches it with stride_q = -1 from add + diag_zero.
         self.mul, self.add, self.fn = mul, add, fn
+        self.diag_zero: Optional[int] = None
 
     def c_struct(self) -> _lib.FlexScoreMod:
         m = _lib.FlexScoreMod(self.kind, self.p0, self.p1, self.i0, 0)
         t = self.mul if self.mul is not None else self.add
-        if t is not None:
+        if t is not None and self.diag_zero is not None:
+            m.add = self.add.data_ptr() + 4 * self.diag_zero
+            m.stride_b, m.stride_h = (t.stride(i) if t.shape[i] > 1 else 0 for i in range(2))
+            m.stride_q = -1
+        elif t is not None:
             m.mul = self.mul.data_ptr() if self.mul is not None else None
             m.add = self.add.data_ptr() if self.add is not None else None
             m.stride_b, m.stride_h, m.stride_q = (t.stride(i) if t.shape[i] > 1 else 0 for i in range(3))
@@ -236,7 +243,13 @@ def affine_score_mod(fn: Callable, B: int, H: int, Lq: int, Lkv: int, device) ->
     mul = None if bool(((mul - 1).abs() <= 1e-6).all()) else torch.broadcast_to(mul, shp).contiguous()
     if add is None and mul is None:
         return IDENTITY
-    return ScoreMod(_lib.SCORE_AFFINE, name=getattr(fn, "__name__", "affine_score_mod"), mul=mul, add=add, fn=fn)
+    spec = ScoreMod(_lib.SCORE_AFFINE, name=getattr(fn, "__name__", "affine_score_mod"), mul=mul, add=add, fn=fn)
+    if (mul is None and add.shape[2] == Lq and Lq > 1 and Lkv > 1
+            and bool(torch.equal(add[:, :, 1:, 1:], add[:, :, :-1, :-1]))):
+        # constant along every diagonal: first column upwards (kv - q = -(Lq-1) .. 0), then first row (1 .. Lkv-1)
+        spec.add = torch.cat([add[:, :, :, 0].flip(-1), add[:, :, 0, 1:]], dim=-1).contiguous()
+        spec.diag_zero = Lq - 1
+    return spec
 
 
 _score_cache: dict = {}

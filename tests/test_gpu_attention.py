@@ -354,7 +354,8 @@ def test_fused_additive_bias_table(dev):
     from flaxattention_amd.core.common import resolve_score_mod
     from flaxattention_amd import _lib
     spec = resolve_score_mod(rel_bias, 6, (2, 6, 200, 200), dev)
-    assert spec.kind == _lib.SCORE_AFFINE and spec.mul is None and spec.add.shape == (1, 6, 200, 200)
+    assert spec.kind == _lib.SCORE_AFFINE and spec.mul is None
+    assert spec.add.shape == (1, 6, 399) and spec.diag_zero == 199      # depends on kv - q only: kept per diagonal
     for dtype, D in ((torch.float16, 64), (torch.bfloat16, 128)):
         print(f"case additive table rel_bias {dtype} D{D}", flush=True)
         run(dev, dtype, 2, 6, 6, 200, 200, D, score=rel_bias, oscore=rel_bias, mask=causal_mask, omask=o_causal_mask,

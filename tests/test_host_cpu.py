@@ -222,12 +222,21 @@ def test_affine_score_mod_lowering_on_cpu():
     def scaled(score, b, h, q_idx, kv_idx):
         return torch.where(q_idx >= kv_idx, score * 0.5, score * 2.0) - 1.5 * b
 
+    # a bias that depends on kv - q only is kept per diagonal: entry (kv - q) + Lq - 1, reached with stride_q = -1
     s = affine_score_mod(rel_table, 2, 3, 6, 7, "cpu")
-    assert s.kind == _lib.SCORE_AFFINE and s.mul is None and tuple(s.add.shape) == (1, 3, 6, 7)
+    assert s.kind == _lib.SCORE_AFFINE and s.mul is None and tuple(s.add.shape) == (1, 3, 12) and s.diag_zero == 5
     c = s.c_struct()
-    assert (c.stride_b, c.stride_h, c.stride_q) == (0, 42, 7) and c.mul is None and c.add == s.add.data_ptr()
+    assert (c.stride_b, c.stride_h, c.stride_q) == (0, 12, -1) and c.mul is None and c.add == s.add.data_ptr() + 4 * 5
     q, kv = torch.arange(6).reshape(6, 1), torch.arange(7).reshape(1, 7)
-    assert torch.equal(s.add[0, 2], table[2][(q - kv).clamp(-4, 4) + 4])
+    assert torch.equal(s.add[0, 2][(kv - q) + 5], table[2][(q - kv).clamp(-4, 4) + 4])
+
+    def per_row(score, b, h, q_idx, kv_idx):   # depends on q and kv separately: stays a dense [.., Lq, Lkv] table
+        return score + table[h.long(), (q_idx % 3 + kv_idx % 4).long()]
+    s = affine_score_mod(per_row, 2, 3, 6, 7, "cpu")
+    assert tuple(s.add.shape) == (1, 3, 6, 7) and s.diag_zero is None
+    c = s.c_struct()
+    assert (c.stride_b, c.stride_h, c.stride_q) == (0, 42, 7) and c.add == s.add.data_ptr()
+    assert torch.equal(s.add[0, 2], table[2][(q % 3 + kv % 4)])
     s = affine_score_mod(scaled, 2, 3, 6, 7, "cpu")
     assert tuple(s.mul.shape) == (2, 1, 6, 7) and torch.equal(s.mul[1, 0], torch.where(q >= kv, 0.5, 2.0))
     assert torch.equal(s.add[1, 0], torch.full((6, 7), -1.5))
