@@ -268,13 +268,16 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
     stamp = _capture_stamp(fn)
     key = (id(fn), H)
     hit = _score_cache.get(key)
-    if hit is not None and hit[0] is fn and _stamp_valid(hit[2]):
+    if hit is not None and not (hit[0] is fn and _stamp_valid(hit[2])):
+        hit = None
+    if hit is not None and hit[1] is not None:
         return hit[1]
-    spec = _probe_score_mod(fn, H, shape, device)
-    if spec is not None:
+    if hit is None:   # (a cached None says: probed before, not one of the families)
+        spec = _probe_score_mod(fn, H, shape, device)
         if stamp is not None:
             _score_cache[key] = (fn, spec, stamp)
-        return spec
+        if spec is not None:
+            return spec
     if shape is not None and device is not None:
         key = (id(fn),) + tuple(shape) + (str(device),)
         hit = _score_cache.get(key)

@@ -172,6 +172,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
         cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
         if (cls == kBlockNone) continue;
       }
+      sm.tile(q_row, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
       // dP starts at -delta, so the accumulator comes out as dP - delta
       float16_t sacc, dpacc, gacc;
 #pragma unroll
@@ -184,7 +185,6 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
         dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + (((2 * s) ^ kz) * 8)), dof[s], dpacc);
       }
       // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
-      sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float s0 = sacc[r], s1 = sacc[r + 1];
@@ -415,6 +415,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       }
       float16_t sacc, dpacc;
       const int ql = qrow_w + 4 * g;  // local row of register 0
+      sm.tileT(q0 + ql, kv_col);      // a table-reading score_mod fetches its entries under the products
 #pragma unroll
       for (int rr = 0; rr < 4; rr++) {
         const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
@@ -432,7 +433,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
       float16_t gacc;
-      sm.tileT(q0 + ql, kv_col);
       if constexpr (KIND == kScoreCheckerboardKv) key_grad = sm.key_grad;
 #pragma unroll
       for (int rr = 0; rr < 4; rr++) {

@@ -149,6 +149,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       int cls = kBlockAll;
       if (masked) cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
       if (cls != kBlockNone) {
+      sm.tile(q_row0, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
       // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
       vec8 kfr[DS], vfr[2][DB];
       {
@@ -184,7 +185,6 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
         const int q_row = q_row0 + 32 * a;
         // ---- score_mod relative to the running reference max, tile mask where needed ----
         m_use[a] = (m_run[a] == -INFINITY) ? 0.f : m_run[a];
-        sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float s0 = sacc[a][r], s1 = sacc[a][r + 1];
