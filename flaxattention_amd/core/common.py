@@ -268,7 +268,7 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
     stamp = _capture_stamp(fn)
     key = (id(fn), H)
     hit = _score_cache.get(key)
-    if hit is not None and not (hit[0] is fn and _stamp_valid(hit[2])):
+    if hit is not None and not (hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp)):
         hit = None
     if hit is not None and hit[1] is not None:
         return hit[1]
@@ -281,7 +281,7 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
     if shape is not None and device is not None:
         key = (id(fn),) + tuple(shape) + (str(device),)
         hit = _score_cache.get(key)
-        if hit is not None and hit[0] is fn and _stamp_valid(hit[2]):
+        if hit is not None and hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp):
             return hit[1]
         spec = affine_score_mod(fn, *shape, device)
         if spec is not None:
@@ -403,16 +403,21 @@ def _eval_mask(fn: Callable, b, h, q, kv) -> torch.Tensor:
     return m.to(torch.bool)
 
 
-def _scan_captures(fn, tensors: list, depth: int = 0) -> bool:
+def _scan_captures(fn, tensors: list, depth: int = 0, scalars: Optional[list] = None) -> bool:
     """Walk what `fn` closes over, defaults to or reads from its globals.  Tensors found on the way are
-    appended to `tensors`; the return value says whether everything else was transparent: numbers, strings,
-    modules, containers of such, and functions that are themselves transparent.  An object of any other kind
-    (an array, a module instance, a bound method) may hold state this walk cannot see."""
+    appended to `tensors` (and numbers / strings to `scalars`, when given); the return value says whether
+    everything else was transparent: modules, containers of such, and functions that are themselves
+    transparent.  An object of any other kind (an array, a module instance, a bound method) may hold state
+    this walk cannot see."""
     import functools
     import types
 
     def plain(x) -> bool:
-        if x is None or isinstance(x, (bool, int, float, complex, str, bytes, types.ModuleType, type)):
+        if x is None or isinstance(x, (types.ModuleType, type)):
+            return True
+        if isinstance(x, (bool, int, float, complex, str, bytes)):
+            if scalars is not None:
+                scalars.append(x)
             return True
         if torch.is_tensor(x):
             tensors.append(x)
@@ -429,7 +434,7 @@ def _scan_captures(fn, tensors: list, depth: int = 0) -> bool:
         if isinstance(x, dict):
             return all([plain(y) for y in x.values()])
         if isinstance(x, (types.FunctionType, types.BuiltinFunctionType, functools.partial)):
-            return _scan_captures(x, tensors, depth + 1)
+            return _scan_captures(x, tensors, depth + 1, scalars)
         return False
 
     if depth > 4:
@@ -459,15 +464,22 @@ def _index_arithmetic_only(fn) -> bool:
 
 def _capture_stamp(fn):
     """What a cached lowering of `fn` depends on besides `fn` itself: the captured tensors with their version
-    counters, or None when `fn` holds state that cannot be seen (then nothing about it may be cached)."""
+    counters and the captured numbers and strings, or None when `fn` holds state that cannot be seen (then
+    nothing about it may be cached)."""
     tensors: list = []
-    if not _scan_captures(fn, tensors):
+    scalars: list = []
+    if not _scan_captures(fn, tensors, 0, scalars):
         return None
-    return [(t, t._version) for t in tensors]
+    return [(t, t._version) for t in tensors] + [(None, tuple(scalars))]
 
 
-def _stamp_valid(stamp) -> bool:
-    return all(t._version == v for t, v in stamp)
+def _stamp_valid(stamp, now=None) -> bool:
+    """`stamp` (taken when a lowering was cached) still describes the callable: the same tensors at the same
+    versions.  `now` is a fresh stamp of the callable (a closure variable may have been rebound to another tensor)."""
+    if now is not None:
+        if len(now) != len(stamp) or any(a[0] is not b[0] for a, b in zip(now, stamp)) or now[-1][1] != stamp[-1][1]:
+            return False
+    return all(t._version == v for t, v in stamp[:-1])
 
 
 def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device,
@@ -573,6 +585,24 @@ def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, de
             return fn
         fn = fn.fn
     Qp, KVp = _pad128(Q), _pad128(KV)
+    # the dense evaluation is remembered per callable, shape and the captured tensors at their versions
+    stamp = _capture_stamp(fn)
+    key = (id(fn), B, H, Q, KV, str(device), real)
+    hit = _mask_cache.get(key)
+    if hit is not None and hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp):
+        return hit[1]
+    spec = _lower_mask_callable(fn, B, H, Q, KV, Qp, KVp, device, real)
+    if stamp is not None:
+        if len(_mask_cache) > 32:
+            _mask_cache.clear()
+        _mask_cache[key] = (fn, spec, stamp)
+    return spec
+
+
+_mask_cache: dict = {}
+
+
+def _lower_mask_callable(fn: Callable, B: int, H: int, Q: int, KV: int, Qp: int, KVp: int, device, real) -> MaskMod:
     m = dense_mask_on_device(fn, B, H, Qp, KVp, device, real=real or (Q, KV))
     name = getattr(fn, "__name__", "mask_mod")
     full_shape = torch.broadcast_shapes(m.shape, (1, 1, Qp, KVp))

@@ -183,6 +183,30 @@ def test_mask_without_block_mask_pallas(dev):
         omask=o_sliding_window(10), score=generate_alibi_bias(2), oscore=o_alibi(2), pallas=True)
 
 
+def test_untagged_mask_lowering_follows_captured_tensor(dev):
+    """flax_attention_pallas(mask_mod=callable): the dense lowering of the callable is reused from call to call
+    and redone when the tensor it captures is updated in place or the closure variable is rebound."""
+    q, k, v = seeded_qkv(1, 2, 2, 96, 96, 64, torch.float16)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    doc_cpu = torch.arange(96) // 24
+    doc = doc_cpu.to(dev)
+
+    def doc_mask(b, h, q_idx, kv_idx):
+        d = doc if q_idx.is_cuda else doc_cpu
+        return d[q_idx.long()] == d[kv_idx.long()]
+    for step in range(3):
+        if step == 1:
+            doc.copy_(torch.arange(96, device=dev) // 40)
+            doc_cpu = torch.arange(96) // 40
+        if step == 2:
+            doc_cpu = torch.arange(96) // 7
+            doc = doc_cpu.to(dev)
+        out = fa.flax_attention_pallas(qd, kd, vd, mask_mod=doc_mask)
+        again = fa.flax_attention_pallas(qd, kd, vd, mask_mod=doc_mask)
+        want = ref_attention(q, k, v, None, doc_mask, strict=True)
+        assert rel_l2(out.cpu(), want) <= 1e-3 and torch.equal(out, again), f"step {step}"
+
+
 def test_bhln_false_layout(dev):
     q, k, v = seeded_qkv(2, 4, 4, 64, 80, 32, torch.float32)
     want = ref_attention(q, k, v, None, o_causal_mask)

@@ -298,10 +298,21 @@ def test_cached_lowerings_follow_captured_tensors():
     table = torch.zeros(4)
     fn = lambda s, b, h, q, kv: s + table[h.long()]   # noqa: E731
     stamp = _capture_stamp(fn)
-    assert stamp is not None and len(stamp) == 1 and stamp[0][0] is table and _stamp_valid(stamp)
+    assert stamp is not None and len(stamp) == 2 and stamp[0][0] is table and _stamp_valid(stamp, _capture_stamp(fn))
     table.add_(1.0)
-    assert not _stamp_valid(stamp)
-    assert _capture_stamp(lambda s, b, h, q, kv: s * 2.0) == []
+    assert not _stamp_valid(stamp, _capture_stamp(fn))
+    assert _capture_stamp(lambda s, b, h, q, kv: s * 2.0) == [(None, ())]
+    window = 3
+    band = lambda b, h, q, kv: q - kv <= window   # noqa: E731
+    stamp = _capture_stamp(band)
+    assert stamp == [(None, (3,))] and _stamp_valid(stamp, _capture_stamp(band))
+    window = 5                                    # a rebound closure variable is a different callable in effect
+    assert not _stamp_valid(stamp, _capture_stamp(band))
+    other = torch.zeros(4)
+    fn2 = lambda s, b, h, q, kv: s + other[h.long()]   # noqa: E731
+    stamp = _capture_stamp(fn2)
+    other = torch.ones(4)                         # rebound to another tensor
+    assert not _stamp_valid(stamp, _capture_stamp(fn2))
 
     class Holder:
         t = torch.ones(2)
