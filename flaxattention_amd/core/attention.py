@@ -276,6 +276,26 @@ class _FlexAttention(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+class _NothingToAttend(torch.autograd.Function):
+    """Inputs with no query rows, batches or heads (empty outputs) or with no keys at all: every row is then a
+    fully masked row, whose output is 0 and whose log-sum-exp is -inf (attention.py:97-104).  Gradients are zero.
+    Nothing is launched; the kernels take positive sizes only."""
+    @staticmethod
+    def forward(ctx, q, k, v):
+        ctx.meta = [(t.shape, t.dtype, t.device) for t in (q, k, v)]
+        out = q.new_zeros(*q.shape[:-1], v.shape[-1])
+        lse2 = torch.full(q.shape[:-1], float("-inf"), dtype=torch.float32, device=q.device)
+        return out, lse2
+
+    @staticmethod
+    def backward(ctx, _d_o, _d_lse):
+        return tuple(torch.zeros(s, dtype=d, device=dev) for s, d, dev in ctx.meta)
+
+
+def _nothing_to_attend(query: Array, key: Array) -> bool:
+    return query.numel() == 0 or key.shape[1] == 0 or key.shape[2] == 0
+
+
 def _as_kernel_layout(t: Array) -> Array:
     return t if t.stride(-1) == 1 else t.contiguous()
 
@@ -345,6 +365,9 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
                 f"but got Hq={Hq} and Hkv={Hkv}."
             )
     _require_device(query, key, value)
+    if _nothing_to_attend(query, key):
+        out, lse2 = _NothingToAttend.apply(query, key, value)
+        return (out, lse2) if return_lse else out
     if score_mod is None:
         score_mod = _identity
     if block_mask is None:
@@ -400,6 +423,9 @@ def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Opt
         sm_scale = 1 / math.sqrt(query.shape[-1])
     if block_mask is not None and mask_mod is not None:
         raise ValueError("pass only one of block_mask= and mask_mod=")
+    if _nothing_to_attend(query, key):
+        out, _ = _NothingToAttend.apply(query, key, value)
+        return out if bhln else out.transpose(1, 2)
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
     out, _ = _FlexAttention.apply(q, k, v, plan)

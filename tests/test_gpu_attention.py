@@ -437,3 +437,24 @@ def test_affine_score_mod_tables(dev):
     q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 64, torch.float16))
     with pytest.raises(NotImplementedError):
         fa.flax_attention(q, k, v, score_mod=quadratic)
+
+
+@pytest.mark.parametrize("shape", [(2, 2, 0, 64, 64), (2, 2, 16, 0, 64), (0, 2, 16, 64, 64), (1, 2, 300, 0, 128)])
+def test_empty_inputs(dev, shape):
+    """No query rows / batches give empty outputs; no keys make every row a fully masked row: output 0,
+    log-sum-exp -inf, zero gradients (attention.py:97-104; tests/attention_test.py:65-129 for the masked form)."""
+    B, H, Lq, Lkv, D = shape
+    print(f"case empty inputs {shape}", flush=True)
+    mk = lambda *s: torch.randn(*s, device=dev, dtype=torch.float16, requires_grad=True)
+    q, k, v = mk(B, H, Lq, D), mk(B, H, Lkv, D), mk(B, H, Lkv, D)
+    out, lse = fa.flax_attention(q, k, v, return_lse=True)
+    assert out.shape == (B, H, Lq, D) and lse.shape == (B, H, Lq) and out.dtype == q.dtype
+    if Lkv == 0:
+        assert out.abs().sum().item() == 0 and bool(torch.isneginf(lse).all())
+    out.sum().backward()
+    for t in (q, k, v):
+        assert t.grad.shape == t.shape and t.grad.abs().sum().item() == 0
+    out_p = fa.flax_attention_pallas(q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), mask_mod=causal_mask, bhln=False)
+    assert out_p.shape == (B, Lq, H, D) and out_p.abs().sum().item() == 0
+    with pytest.raises(ValueError):   # the validators still run first
+        fa.flax_attention(q, k.float(), v)
