@@ -318,3 +318,9 @@ def test_cached_lowerings_follow_captured_tensors():
         t = torch.ones(2)
     holder = Holder()
     assert _capture_stamp(lambda s, b, h, q, kv: s + holder.t[0]) is None   # state that cannot be seen: never cached
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU; asking for more ends with a message instead of a number."""
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
