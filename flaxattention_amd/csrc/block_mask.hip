@@ -66,28 +66,38 @@ __global__ __launch_bounds__(kClassifyThreads) void classify_tiles_kernel(
   }
 }
 
+// The four ordered lists of a block mask (partial / full, by query block / by key block) come from one
+// launch: blockIdx.y names the list.
+struct OrderJob {
+  const int8_t* flags;
+  int32_t* num;
+  int32_t* idx;
+  int nrows, ncols, row_stride, col_stride;
+};
+struct OrderJobs { OrderJob job[4]; };
+
 // One wave per output row.  Reads flags[bh][r*row_stride + c*col_stride] for
 // c in [0, ncols) and writes num[bh][r] and idx[bh][r][0..ncols).
-__global__ __launch_bounds__(256) void order_rows_kernel(const int8_t* __restrict__ flags, int nrows,
-                                                         int ncols, long long mat_stride,
-                                                         int row_stride, int col_stride,
-                                                         int32_t* __restrict__ num,
-                                                         int32_t* __restrict__ idx, long long total_rows) {
+__global__ __launch_bounds__(256) void order_rows_kernel(OrderJobs jobs, long long mat_stride, long long n_bh) {
+  const OrderJob& jb = jobs.job[blockIdx.y];
+  if (!jb.num && !jb.idx) return;
+  const int nrows = jb.nrows, ncols = jb.ncols;
   const int lane = threadIdx.x & 63;
   const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (row >= total_rows) return;
+  if (row >= n_bh * nrows) return;
   const long long bh = row / nrows;
   const int r = (int)(row % nrows);
-  const int8_t* f = flags + bh * mat_stride + (long long)r * row_stride;
+  const int8_t* f = jb.flags + bh * mat_stride + (long long)r * jb.row_stride;
+  const int col_stride = jb.col_stride;
   int count = 0;
   for (int c0 = 0; c0 < ncols; c0 += 64) {
     int c = c0 + lane;
     bool sel = (c < ncols) && f[(long long)c * col_stride] != 0;
     count += __popcll(__ballot(sel));
   }
-  if (num && lane == 0) num[row] = count;
-  if (!idx) return;
-  int32_t* out = idx + row * ncols;
+  if (jb.num && lane == 0) jb.num[row] = count;
+  if (!jb.idx) return;
+  int32_t* out = jb.idx + row * ncols;
   int before_sel = 0, before_uns = 0;
   const unsigned long long lt = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
   for (int c0 = 0; c0 < ncols; c0 += 64) {
@@ -134,22 +144,30 @@ extern "C" int flexattn_block_mask_build(const FlexMask* mask, int32_t B, int32_
   size_t n = (size_t)B * H * nq * nkv;
   int8_t* partial = (int8_t*)workspace;
   int8_t* full = partial + (n + 255) / 256 * 256;
-  dim3 grid(nkv, nq, B * H);
+  // a band mask (or a bitmap broadcast over batch and head) does not look at (b, h): its tiles are classified once
+  // and every (b, h) orders the same flags
+  const bool uniform = mask->kind == FLEX_MASK_BAND || (mask->bits_stride_b == 0 && mask->bits_stride_h == 0);
+  dim3 grid(nkv, nq, uniform ? 1 : B * H);
   hipLaunchKernelGGL(classify_tiles_kernel, grid, dim3(kClassifyThreads), 0, stream, *mask, H, nq, nkv, qb, kvb, partial, full);
-  const long long mat = (long long)nq * nkv;
-  auto order = [&](const int8_t* flags, bool transposed, int32_t* num, int32_t* idx) {
-    if (!num && !idx) return;
-    int nrows = transposed ? nkv : nq, ncols = transposed ? nq : nkv;
-    int rs = transposed ? 1 : nkv, cs = transposed ? nkv : 1;
-    long long total_rows = (long long)B * H * nrows;
-    int waves = 4;
-    long long blocks = (total_rows + waves - 1) / waves;
-    hipLaunchKernelGGL(order_rows_kernel, dim3((unsigned)blocks), dim3(64 * waves), 0, stream, flags, nrows, ncols, mat, rs, cs, num, idx, total_rows);
+  const long long mat = uniform ? 0 : (long long)nq * nkv;
+  OrderJobs jobs;
+  auto job = [&](int at, const int8_t* flags, bool transposed, int32_t* num, int32_t* idx) {
+    OrderJob& j = jobs.job[at];
+    j.flags = flags; j.num = num; j.idx = idx;
+    j.nrows = transposed ? nkv : nq; j.ncols = transposed ? nq : nkv;
+    j.row_stride = transposed ? 1 : nkv; j.col_stride = transposed ? nkv : 1;
   };
-  order(partial, false, kv_num, kv_idx);
-  order(full, false, full_kv_num, full_kv_idx);
-  order(partial, true, q_num, q_idx);
-  order(full, true, full_q_num, full_q_idx);
+  job(0, partial, false, kv_num, kv_idx);
+  job(1, full, false, full_kv_num, full_kv_idx);
+  job(2, partial, true, q_num, q_idx);
+  job(3, full, true, full_q_num, full_q_idx);
+  const bool by_kv = kv_num || kv_idx || full_kv_num || full_kv_idx, by_q = q_num || q_idx || full_q_num || full_q_idx;
+  if (by_kv || by_q) {
+    const int waves = 4;
+    const long long most_rows = (long long)B * H * (by_q ? (by_kv ? (nq > nkv ? nq : nkv) : nkv) : nq);
+    const long long blocks = (most_rows + waves - 1) / waves;
+    hipLaunchKernelGGL(order_rows_kernel, dim3((unsigned)blocks, 4), dim3(64 * waves), 0, stream, jobs, mat, (long long)B * H);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { flex_set_error("block_mask_build: launch failed: %s", hipGetErrorString(e)); return 2; }
   return 0;
