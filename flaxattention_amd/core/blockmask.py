@@ -293,10 +293,8 @@ def build_lists(spec: MaskMod, B: int, H: int, nq: int, nkv: int, q_block: int, 
     return out
 
 
-def _create_empty_block_mask(query: Array, key: Array) -> BlockMask:
-    """Default block mask: one block spanning everything, noop mask
-    (blockmask.py:240-250)."""
-    dev = query.device
+@functools.lru_cache(maxsize=None)
+def _empty_block_mask_on(dev: torch.device) -> BlockMask:
     bm = BlockMask.from_kv_blocks(
         kv_num_blocks=torch.ones([1, 1, 1], dtype=torch.int32, device=dev),
         kv_indices=torch.zeros([1, 1, 1, 1], dtype=torch.int32, device=dev),
@@ -304,6 +302,13 @@ def _create_empty_block_mask(query: Array, key: Array) -> BlockMask:
     )
     bm.spec = noop_mask
     return bm
+
+
+def _create_empty_block_mask(query: Array, key: Array) -> BlockMask:
+    """Default block mask: one block spanning everything, noop mask
+    (blockmask.py:240-250).  It depends on nothing but the device and nothing writes to it, so one object per
+    device serves every call (building it takes a dozen small launches)."""
+    return _empty_block_mask_on(query.device)
 
 
 def create_block_mask(mask_mod: _mask_mod_signature, B: Optional[int], H: Optional[int], Q_LEN: int, KV_LEN: int,
