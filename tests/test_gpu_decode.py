@@ -126,3 +126,34 @@ def test_decode_in_chunks_of_64_rows(dev):
     assert max_abs(lse.cpu(), want_lse) <= 2e-2
     ref = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, kernel_options={"decode": False})
     assert max_abs(out.cpu(), ref.cpu()) <= 2e-3
+
+
+@pytest.mark.parametrize("Lq", [1, 200])
+def test_calls_replay_from_a_captured_graph(dev, Lq):
+    """Nothing on the path synchronises, allocates outside the caller's allocator or records a memset, so a serving
+    loop can capture a call (here one decode call, and a 200-row query served as four decode calls) in a HIP graph
+    and replay it.  Every replay, with eager work of the same kind between the replays, gives the eager call's bits."""
+    print(f"case graph capture q_len {Lq}", flush=True)
+    B, H, Lkv, D = 2, 8, 4096, 64
+    g0 = torch.Generator(device="cpu").manual_seed(0)
+    mk = lambda *s: torch.randn(*s, generator=g0, dtype=torch.float32).to(torch.float16).to(dev)
+    K, V, q_static = mk(B, H, Lkv, D), mk(B, H, Lkv, D), mk(B, H, Lq, D)
+    bm = fa.create_block_mask(offset_causal_mask(Lkv - Lq), 1, 1, Lq, Lkv, device=dev)
+    call = lambda q: fa.flax_attention(q, K, V, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True)
+    side = torch.cuda.Stream()   # default priority; warm-up off the default stream as graph capture asks
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            call(q_static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static, lse_static = call(q_static)
+    for i in range(4):
+        q_new = mk(B, H, Lq, D)
+        q_static.copy_(q_new)
+        graph.replay()
+        eager, eager_lse = call(q_new)
+        torch.cuda.synchronize()
+        assert torch.equal(out_static, eager) and torch.equal(lse_static, eager_lse), f"replay {i} differs from the eager call"
