@@ -276,6 +276,12 @@ class _FlexAttention(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+def _attend(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
+        return _FlexAttention.apply(q, k, v, plan)
+    return _run_fwd(plan, q, k, v)   # nothing to differentiate: no need to pay for the autograd wrapper
+
+
 class _NothingToAttend(torch.autograd.Function):
     """Inputs with no query rows, batches or heads (empty outputs) or with no keys at all: every row is then a
     fully masked row, whose output is 0 and whose log-sum-exp is -inf (attention.py:97-104).  Gradients are zero.
@@ -338,7 +344,7 @@ def math_attention(query: Array, key: Array, value: Array, score_mod: Callable, 
     opts = dict(kernel_options or {})
     opts.setdefault("strict", True)
     plan = _make_plan(q, k, v, score_mod, None, mask_mod, scale, opts)
-    return _FlexAttention.apply(q, k, v, plan)
+    return _attend(plan, q, k, v)
 
 
 def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_score_mod_signature] = None,
@@ -376,7 +382,7 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
         scale = 1.0 / math.sqrt(query.shape[-1])
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
-    out, lse2 = _FlexAttention.apply(q, k, v, plan)
+    out, lse2 = _attend(plan, q, k, v)
     out = out[..., :value.shape[-1]]
     if return_lse:
         return out, lse2 * math.log(2.0)
@@ -428,6 +434,6 @@ def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Opt
         return out if bhln else out.transpose(1, 2)
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
-    out, _ = _FlexAttention.apply(q, k, v, plan)
+    out, _ = _attend(plan, q, k, v)
     out = out[..., :value.shape[-1]]
     return out if bhln else out.transpose(1, 2)
