@@ -31,7 +31,9 @@ class FlexScoreMod(C.Structure):
 class FlexMask(C.Structure):
     _fields_ = [("kind", C.c_int32), ("lo", C.c_int32), ("hi", C.c_int32), ("sink", C.c_int32),
                 ("q_offset", C.c_int32), ("pad_", C.c_int32), ("bits", C.c_void_p),
-                ("bits_stride_b", C.c_int64), ("bits_stride_h", C.c_int64), ("bits_stride_q", C.c_int64)]
+                ("bits_stride_b", C.c_int64), ("bits_stride_h", C.c_int64), ("bits_stride_q", C.c_int64),
+                ("bits_t", C.c_void_p),
+                ("bits_t_stride_b", C.c_int64), ("bits_t_stride_h", C.c_int64), ("bits_t_stride_kv", C.c_int64)]
 
 
 class FlexTileLists(C.Structure):

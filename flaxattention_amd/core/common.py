@@ -308,9 +308,11 @@ class MaskMod:
     or a packed bitmap made from an arbitrary callable (kind BITS)."""
 
     def __init__(self, lo: int = INT_MIN, hi: int = INT_MAX, sink: int = -1, q_offset: int = 0,
-                 name: str = "mask_mod", bits: Optional[torch.Tensor] = None, fn: Optional[Callable] = None):
+                 name: str = "mask_mod", bits: Optional[torch.Tensor] = None, fn: Optional[Callable] = None,
+                 bits_t: Optional[torch.Tensor] = None):
         self.lo, self.hi, self.sink, self.q_offset = int(lo), int(hi), int(sink), int(q_offset)
         self.bits = bits      # int32 [Bm, Hm, Qp, KVw] on the device, or None
+        self.bits_t = bits_t  # the same bitmap packed along the query axis, int32 [Bm, Hm, KVp, Qw], or None
         self.fn = fn          # the callable a bitmap was made from
         self.__name__ = name
 
@@ -335,6 +337,12 @@ class MaskMod:
             m.bits_stride_b = 0 if Bm == 1 else Hm * Qp * W
             m.bits_stride_h = 0 if Hm == 1 else Qp * W
             m.bits_stride_q = W
+            if self.bits_t is not None:
+                _, _, KVp, Wq = self.bits_t.shape
+                m.bits_t = self.bits_t.data_ptr()
+                m.bits_t_stride_b = 0 if Bm == 1 else Hm * KVp * Wq
+                m.bits_t_stride_h = 0 if Hm == 1 else KVp * Wq
+                m.bits_t_stride_kv = Wq
         return m
 
     def __call__(self, b, h, q_idx, kv_idx):
@@ -614,5 +622,6 @@ def _lower_mask_callable(fn: Callable, B: int, H: int, Q: int, KV: int, Qp: int,
             band.__name__ = name
             return band
         m = m[:1, :1]
-    bits = pack_bits(m.contiguous())
-    return MaskMod(name=name, bits=bits, fn=fn)
+    # packed along the key axis for the kernels whose lanes own a query row, and along the query axis for the
+    # dK/dV kernel, whose lanes own a key
+    return MaskMod(name=name, bits=pack_bits(m.contiguous()), fn=fn, bits_t=pack_bits(m.transpose(-1, -2).contiguous()))

@@ -143,11 +143,15 @@ struct MaskEval {
   int32_t kind, lo, hi, sink, q_offset;
   const uint32_t* bits_bh;  // bitmap row base of the current (b, h)
   int64_t stride_q;
+  const uint32_t* bits_t_bh;  // the same bitmap packed along the query axis (may be null)
+  int64_t stride_kv;
 
   __device__ __forceinline__ MaskEval(const FlexMask& m, int b, int h) {
     kind = m.kind; lo = m.lo; hi = m.hi; sink = m.sink; q_offset = m.q_offset;
     bits_bh = m.bits ? m.bits + b * m.bits_stride_b + h * m.bits_stride_h : nullptr;
     stride_q = m.bits_stride_q;
+    bits_t_bh = m.bits_t ? m.bits_t + b * m.bits_t_stride_b + h * m.bits_t_stride_h : nullptr;
+    stride_kv = m.bits_t_stride_kv;
   }
   __device__ __forceinline__ bool operator()(int q, int kv) const {
     if (kind == FLEX_MASK_BAND) {

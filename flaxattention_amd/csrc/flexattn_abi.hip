@@ -64,7 +64,7 @@ static int check_launch(const char* who) {
   return 0;
 }
 
-extern "C" int flexattn_abi_version(void) { return 1; }
+extern "C" int flexattn_abi_version(void) { return 2; }
 extern "C" const char* flexattn_last_error(void) { return g_err; }
 
 extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t which, int32_t* qb, int32_t* kvb) {

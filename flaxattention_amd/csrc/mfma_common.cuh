@@ -322,6 +322,16 @@ __device__ __forceinline__ void mask_block_kv(float16_t& x, const FlexMask& m, c
       const bool vis = (off >= lo_off) & (off <= hi_off);
       x[r] = vis ? x[r] : -INFINITY;
     }
+  } else if (visible.ev.bits_t_bh) {
+    // query-packed copy: the 32 query rows of this block (qb = 32-aligned row + 4*g) are one word of key kv
+    const uint32_t w = kv < Lkv ? visible.ev.bits_t_bh[(int64_t)kv * visible.ev.stride_kv + (qb >> 5)] >> (qb & 31) : 0u;
+    const int up = Lq - 1 - qb;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int off = acc_row(r);
+      const bool vis = ((w >> off) & 1u) & (off <= up);
+      x[r] = vis ? x[r] : -INFINITY;
+    }
   } else {
 #pragma unroll
     for (int r = 0; r < 16; r++) {

@@ -63,7 +63,11 @@ typedef struct FlexScoreMod {
  *     d = q_idx + q_offset - kv_idx
  *     visible = (d >= lo) && (d <= hi || kv_idx <= sink)
  * FLEX_MASK_BITS reads a packed bitmap produced from an arbitrary Python
- * callable: bit (kv & 31) of word bits[b*sb + h*sh + q*sq + (kv >> 5)].  */
+ * callable: bit (kv & 31) of word bits[b*sb + h*sh + q*sq + (kv >> 5)].
+ * bits_t is an optional second copy of the same bitmap packed along the query
+ * axis: bit (q & 31) of word bits_t[b*tb + h*th + kv*tkv + (q >> 5)].  The
+ * dK/dV kernel, whose lanes own keys, then reads one word per 32x32 block
+ * instead of one per entry; without it (NULL) the result is the same.  */
 enum FlexMaskKind { FLEX_MASK_BAND = 0, FLEX_MASK_BITS = 1 };
 
 typedef struct FlexMask {
@@ -72,6 +76,8 @@ typedef struct FlexMask {
   int32_t pad_;
   const uint32_t* bits;
   int64_t bits_stride_b, bits_stride_h, bits_stride_q; /* in 32-bit words */
+  const uint32_t* bits_t;
+  int64_t bits_t_stride_b, bits_t_stride_h, bits_t_stride_kv; /* in 32-bit words */
 } FlexMask;
 
 /* numerics switches (OR-ed into FlexAttnParams.flags) */

@@ -458,3 +458,39 @@ def test_empty_inputs(dev, shape):
     assert out_p.shape == (B, Lq, H, D) and out_p.abs().sum().item() == 0
     with pytest.raises(ValueError):   # the validators still run first
         fa.flax_attention(q, k.float(), v)
+
+
+def test_bitmap_mask_with_and_without_query_packed_copy(dev):
+    """A bitmap mask carries a second copy packed along the query axis for the dK/dV kernel (one word per 32 x 32
+    block instead of one per entry).  A caller of the C ABI may leave it out: the gradients are the same bits."""
+    from flaxattention_amd.core.common import resolve_mask_mod
+    print("case bitmap with / without query-packed copy", flush=True)
+    B, H, Lq, Lkv, D = 2, 2, 200, 330, 64
+    g = torch.Generator(device="cpu").manual_seed(5)
+    keep = (torch.rand(B, 1, Lq, Lkv, generator=g) < 0.5)
+    keep[..., 0] = True
+    keep_dev = keep.to(dev)
+
+    def mask(b, h, q_idx, kv_idx):
+        t = keep_dev if q_idx.is_cuda else keep
+        return t[b.long(), 0, q_idx.long(), kv_idx.long()]
+    spec = resolve_mask_mod(mask, B, H, Lq, Lkv, dev)
+    assert spec.bits is not None and spec.bits_t is not None
+    assert spec.bits_t.shape[-2] == spec.bits.shape[-1] * 32 and spec.bits_t.shape[-1] * 32 == spec.bits.shape[-2]
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(torch.float16).to(dev)
+    q, k, v, d_o = mk(B, H, Lq, D), mk(B, H, Lkv, D), mk(B, H, Lkv, D), mk(B, H, Lq, D)
+    grads = []
+    for with_copy in (True, False):
+        m = spec if with_copy else type(spec)(name="no_copy", bits=spec.bits, fn=spec.fn)
+        qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+        out = fa.flax_attention_pallas(qd, kd, vd, mask_mod=m)
+        out.backward(d_o)
+        grads.append((out.detach(), qd.grad, kd.grad, vd.grad))
+    for a, b_ in zip(*grads):
+        assert torch.equal(a, b_)
+    # and against the oracle
+    want = ref_attention(q.cpu(), k.cpu(), v.cpu(), None, mask, strict=True)
+    assert rel_l2(grads[0][0].cpu(), want) <= 1e-3
+    wq, wk, wv = ref_attention_bwd(q.cpu(), k.cpu(), v.cpu(), d_o.cpu(), None, mask, strict=True)
+    for got, w in zip(grads[0][1:], (wq, wk, wv)):
+        assert rel_l2(got.cpu(), w) <= 1e-3
