@@ -33,7 +33,9 @@ class FlexMask(C.Structure):
                 ("q_offset", C.c_int32), ("pad_", C.c_int32), ("bits", C.c_void_p),
                 ("bits_stride_b", C.c_int64), ("bits_stride_h", C.c_int64), ("bits_stride_q", C.c_int64),
                 ("bits_t", C.c_void_p),
-                ("bits_t_stride_b", C.c_int64), ("bits_t_stride_h", C.c_int64), ("bits_t_stride_kv", C.c_int64)]
+                ("bits_t_stride_b", C.c_int64), ("bits_t_stride_h", C.c_int64), ("bits_t_stride_kv", C.c_int64),
+                ("blk", C.c_void_p),
+                ("blk_stride_b", C.c_int64), ("blk_stride_h", C.c_int64), ("blk_stride_q", C.c_int64)]
 
 
 class FlexTileLists(C.Structure):

@@ -309,10 +309,11 @@ class MaskMod:
 
     def __init__(self, lo: int = INT_MIN, hi: int = INT_MAX, sink: int = -1, q_offset: int = 0,
                  name: str = "mask_mod", bits: Optional[torch.Tensor] = None, fn: Optional[Callable] = None,
-                 bits_t: Optional[torch.Tensor] = None):
+                 bits_t: Optional[torch.Tensor] = None, blk: Optional[torch.Tensor] = None):
         self.lo, self.hi, self.sink, self.q_offset = int(lo), int(hi), int(sink), int(q_offset)
         self.bits = bits      # int32 [Bm, Hm, Qp, KVw] on the device, or None
         self.bits_t = bits_t  # the same bitmap packed along the query axis, int32 [Bm, Hm, KVp, Qw], or None
+        self.blk = blk        # class of every aligned 32 x 32 block, int8 [Bm, Hm, Qp/32, KVp/32], or None
         self.fn = fn          # the callable a bitmap was made from
         self.__name__ = name
 
@@ -343,6 +344,12 @@ class MaskMod:
                 m.bits_t_stride_b = 0 if Bm == 1 else Hm * KVp * Wq
                 m.bits_t_stride_h = 0 if Hm == 1 else KVp * Wq
                 m.bits_t_stride_kv = Wq
+            if self.blk is not None:
+                _, _, nqb, nkb = self.blk.shape
+                m.blk = self.blk.data_ptr()
+                m.blk_stride_b = 0 if Bm == 1 else Hm * nqb * nkb
+                m.blk_stride_h = 0 if Hm == 1 else nqb * nkb
+                m.blk_stride_q = nkb
         return m
 
     def __call__(self, b, h, q_idx, kv_idx):
@@ -576,6 +583,17 @@ def pack_bits(mask: torch.Tensor) -> torch.Tensor:
     return words.to(torch.int32).contiguous()
 
 
+def block_classes(mask: torch.Tensor) -> torch.Tensor:
+    """bool [..., Q, KV] (both multiples of 32) -> int8 [..., Q/32, KV/32]: 1 where a 32 x 32 block is entirely set,
+    2 where it is entirely clear, 0 otherwise (the kernels' kBlockAll / kBlockNone / kBlockMixed)."""
+    *lead, Q, KV = mask.shape
+    count = mask.reshape(*lead, Q // 32, 32, KV // 32, 32).sum(dim=(-3, -1), dtype=torch.int32)
+    cls = torch.zeros_like(count, dtype=torch.int8)
+    cls[count == 1024] = 1
+    cls[count == 0] = 2
+    return cls.contiguous()
+
+
 def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, device,
                      real: Optional[Tuple[int, int]] = None) -> MaskMod:
     """Lower a mask_mod callable to a kernel functor that is exact on the
@@ -624,4 +642,5 @@ def _lower_mask_callable(fn: Callable, B: int, H: int, Q: int, KV: int, Qp: int,
         m = m[:1, :1]
     # packed along the key axis for the kernels whose lanes own a query row, and along the query axis for the
     # dK/dV kernel, whose lanes own a key
-    return MaskMod(name=name, bits=pack_bits(m.contiguous()), fn=fn, bits_t=pack_bits(m.transpose(-1, -2).contiguous()))
+    return MaskMod(name=name, bits=pack_bits(m.contiguous()), fn=fn, bits_t=pack_bits(m.transpose(-1, -2).contiguous()),
+                   blk=block_classes(m))

@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
       // entirely hidden (nothing to do)
       int cls = kBlockAll;
       if (masked) {
-        cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
         if (cls == kBlockNone) continue;
       }
       sm.tile(q_row, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
@@ -410,7 +410,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       const int qrow_w = qs * 32;
       int cls = kBlockAll;
       if (masked) {
-        cls = band_block_class(p.mask, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
+        cls = block_class(p.mask, visible, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
         if (cls == kBlockNone) continue;
       }
       float16_t sacc, dpacc;

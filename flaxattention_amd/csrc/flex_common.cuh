@@ -145,6 +145,8 @@ struct MaskEval {
   int64_t stride_q;
   const uint32_t* bits_t_bh;  // the same bitmap packed along the query axis (may be null)
   int64_t stride_kv;
+  const int8_t* blk_bh;  // class of every aligned 32x32 block of the bitmap (may be null)
+  int64_t blk_stride_q;
 
   __device__ __forceinline__ MaskEval(const FlexMask& m, int b, int h) {
     kind = m.kind; lo = m.lo; hi = m.hi; sink = m.sink; q_offset = m.q_offset;
@@ -152,6 +154,8 @@ struct MaskEval {
     stride_q = m.bits_stride_q;
     bits_t_bh = m.bits_t ? m.bits_t + b * m.bits_t_stride_b + h * m.bits_t_stride_h : nullptr;
     stride_kv = m.bits_t_stride_kv;
+    blk_bh = m.blk ? m.blk + b * m.blk_stride_b + h * m.blk_stride_h : nullptr;
+    blk_stride_q = m.blk_stride_q;
   }
   __device__ __forceinline__ bool operator()(int q, int kv) const {
     if (kind == FLEX_MASK_BAND) {

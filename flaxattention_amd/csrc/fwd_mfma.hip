@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
       // entirely hidden (the step is skipped)
       int cls = kBlockAll;
-      if (masked) cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+      if (masked) cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
       if (cls != kBlockNone) {
       sm.tile(q_row0, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
       // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
           // most 32x32 blocks of a partial tile are entirely visible or entirely hidden
-          const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
+          const int cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_opaque - i32),
                                            __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
           if (cls == kBlockNone) fill_masked(s_cur);
           else if (cls == kBlockMixed) mask_block_q(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);

@@ -264,6 +264,18 @@ __device__ __forceinline__ int band_block_class(const FlexMask& m, int q_first, 
   if (dmax < lo || (dmin > hi && kv_first > snk) || kv_first >= Lkv || q_first >= Lq) return kBlockNone;
   return kBlockMixed;
 }
+// The same for any mask: a bitmap answers from its table of block classes when it carries one.
+// q_first and kv_first are multiples of 32.  The table describes the padded index range, so a
+// block that reaches past the real lengths is never reported as entirely visible.
+__device__ __forceinline__ int block_class(const FlexMask& m, const Mask2& visible, int q_first, int kv_first, int Lq,
+                                           int Lkv) {
+  if (m.kind == FLEX_MASK_BAND) return band_block_class(m, q_first, kv_first, Lq, Lkv);
+  if (!visible.ev.blk_bh) return kBlockMixed;
+  if (kv_first >= Lkv || q_first >= Lq) return kBlockNone;
+  const int c = visible.ev.blk_bh[(int64_t)(q_first >> 5) * visible.ev.blk_stride_q + (kv_first >> 5)];
+  if (c == kBlockAll && (kv_first + 31 >= Lkv || (Lq - 31 <= q_first))) return kBlockMixed;
+  return c;
+}
 __device__ __forceinline__ void fill_masked(float16_t& x) {
 #pragma unroll
   for (int r = 0; r < 16; r++) x[r] = -INFINITY;

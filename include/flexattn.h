@@ -67,7 +67,12 @@ typedef struct FlexScoreMod {
  * bits_t is an optional second copy of the same bitmap packed along the query
  * axis: bit (q & 31) of word bits_t[b*tb + h*th + kv*tkv + (q >> 5)].  The
  * dK/dV kernel, whose lanes own keys, then reads one word per 32x32 block
- * instead of one per entry; without it (NULL) the result is the same.  */
+ * instead of one per entry; without it (NULL) the result is the same.
+ * blk, also optional, classifies every aligned 32x32 block of the bitmap:
+ * blk[b*kb + h*kh + (q >> 5)*kq + (kv >> 5)] = 0 (some entries set), 1 (all
+ * set) or 2 (none set).  Inside a partial tile the fused kernels then skip
+ * hidden blocks and the mask evaluation of fully visible ones, as they do
+ * for band masks by arithmetic.  */
 enum FlexMaskKind { FLEX_MASK_BAND = 0, FLEX_MASK_BITS = 1 };
 
 typedef struct FlexMask {
@@ -78,6 +83,8 @@ typedef struct FlexMask {
   int64_t bits_stride_b, bits_stride_h, bits_stride_q; /* in 32-bit words */
   const uint32_t* bits_t;
   int64_t bits_t_stride_b, bits_t_stride_h, bits_t_stride_kv; /* in 32-bit words */
+  const int8_t* blk;
+  int64_t blk_stride_b, blk_stride_h, blk_stride_q; /* in bytes */
 } FlexMask;
 
 /* numerics switches (OR-ed into FlexAttnParams.flags) */

@@ -324,3 +324,23 @@ def test_bench_refuses_more_than_one_gpu():
     """The benchmark measures one GPU; asking for more ends with a message instead of a number."""
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=300)
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_block_classes_of_a_bitmap():
+    """The table the fused kernels consult inside partial tiles: 1 = block entirely visible, 2 = entirely hidden."""
+    from flaxattention_amd.core.common import block_classes
+    g = torch.Generator().manual_seed(3)
+    m = torch.rand(2, 1, 96, 128, generator=g) < 0.5
+    m[0, 0, 32:64, 64:96] = True
+    m[1, 0, 0:32, 0:32] = False
+    m[1, 0, 64:96, 96:128] = True
+    m[1, 0, 95, 127] = False      # one hidden entry: mixed
+    cls = block_classes(m)
+    assert cls.shape == (2, 1, 3, 4) and cls.dtype == torch.int8
+    for b in range(2):
+        for i in range(3):
+            for j in range(4):
+                blk = m[b, 0, 32 * i:32 * i + 32, 32 * j:32 * j + 32]
+                want = 1 if bool(blk.all()) else (2 if not bool(blk.any()) else 0)
+                assert int(cls[b, 0, i, j]) == want
+    assert int(cls[0, 0, 1, 2]) == 1 and int(cls[1, 0, 0, 0]) == 2 and int(cls[1, 0, 2, 3]) == 0
