@@ -262,7 +262,9 @@ template <int D> struct DkvShape {
   static constexpr int kStages = D == 64 ? 2 : 1;  // LDS stages of the query-side tiles
 };
 
-template <typename T, int D, int KIND, bool ROUND_S>
+// BITS: the mask is a bitmap.  Band masks get an instantiation of their own, without the bitmap code: with it in the
+// same function the compiler allocates registers differently and the unmasked path runs 5 % slower.
+template <typename T, int D, int KIND, bool ROUND_S, bool BITS>
 __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                                const T* __restrict__ k, const T* __restrict__ v,
                                                                const float* __restrict__ lse2,
@@ -314,7 +316,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
   for (int gi = 0; gi < G; gi++) {
     const int h = hk * G + gi;
     sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
-    Mask2 visible(p.mask, b, h, p.Lkv);
     const int32_t* full_idx = nullptr;
     const int32_t* part_idx = nullptr;
     int n_full, n_part = 0;
@@ -410,7 +411,12 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       const int qrow_w = qs * 32;
       int cls = kBlockAll;
       if (masked) {
-        cls = block_class(p.mask, visible, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
+        if constexpr (BITS) {
+          const Mask2 visible(p.mask, b, h, p.Lkv);
+          cls = block_class(p.mask, visible, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
+        } else {
+          cls = band_block_class(p.mask, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
+        }
         if (cls == kBlockNone) continue;
       }
       float16_t sacc, dpacc;
@@ -453,7 +459,8 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       if (cls == kBlockMixed) {
         int q_opaque = q0 + ql, kv_opaque = kv_col;
         asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));  // keeps the mask arithmetic behind this branch
-        mask_block_kv(sacc, p.mask, visible, q_opaque, kv_opaque, p.Lq, p.Lkv);
+        const Mask2 visible(p.mask, b, h, p.Lkv);
+        mask_block_kv<BITS>(sacc, p.mask, visible, q_opaque, kv_opaque, p.Lq, p.Lkv);
       }
       vec8 pf[2], dsf[2];
 #pragma unroll
@@ -513,10 +520,33 @@ template <int D, typename T> constexpr size_t dkv_smem() {
   return DkvShape<D>::kStages * ((size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
 }
 
+template <typename T, int D, int KIND, bool RS, bool BITS>
+static int launch_dkv_as(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
+                         void* dk, void* dv, float* delta, hipStream_t s) {
+  constexpr size_t sm = dkv_smem<D, T>();
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS, BITS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
+    if (e != hipSuccess) return 2;
+    attr_set = true;
+  }
+  const int nkt = (p.Lkv + kListBN - 1) / kListBN;
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS, BITS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p,
+                     (const T*)q, (const T*)k, (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
+  return 0;
+}
+template <typename T, int D, int KIND, bool RS>
+static int launch_dkv(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
+                      void* dk, void* dv, float* delta, hipStream_t s) {
+  if (p.mask.kind == FLEX_MASK_BITS) return launch_dkv_as<T, D, KIND, RS, true>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
+  return launch_dkv_as<T, D, KIND, RS, false>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
+}
+
 template <typename T, int D, int KIND, bool RS>
 static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  const int nqt = (p.Lq + kBM - 1) / kBM, nkt = (p.Lkv + kListBN - 1) / kListBN;
+  const int nqt = (p.Lq + kBM - 1) / kBM;
   if (!(p.flags & FLEX_BWD_ONLY_DKV)) {
     if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.p0 > 0.f && p.score.p1 > 0.f) {
       // positive factors: the derivative folds into the exponent
@@ -529,31 +559,12 @@ static int launch_one(const FlexAttnParams& p, const void* q, const void* k, con
     }
   }
   if (p.flags & FLEX_BWD_ONLY_DQ) return 0;
-  constexpr size_t sm = dkv_smem<D, T>();
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
-    if (e != hipSuccess) return 2;
-    attr_set = true;
-  }
   if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.i0) {
     // keyed on the key index: the derivative is constant along a lane's dK row
     constexpr int KV = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardKv : KIND;
-    static bool attr_kv = false;
-    if (!attr_kv) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KV, RS>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
-      if (e != hipSuccess) return 2;
-      attr_kv = true;
-    }
-    hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KV, RS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p, (const T*)q,
-                       (const T*)k, (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
-    return 0;
+    return launch_dkv<T, D, KV, RS>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
   }
-  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p, (const T*)q, (const T*)k,
-                     (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
-  return 0;
+  return launch_dkv<T, D, KIND, RS>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
 }
 
 template <typename T, int D, int KIND>

@@ -320,9 +320,11 @@ __device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m
 }
 
 // Lane owns key kv; register r holds query qb + acc_row(r) (qb already includes 4*g).
+// BITS = false: the caller knows that the mask is a band mask.
+template <bool BITS>
 __device__ __forceinline__ void mask_block_kv(float16_t& x, const FlexMask& m, const Mask2& visible, int qb, int kv,
                                               int Lq, int Lkv) {
-  if (m.kind == FLEX_MASK_BAND) {
+  if (!BITS || m.kind == FLEX_MASK_BAND) {
     const int dq = qb + m.q_offset - kv;                          // d = dq + off
     const int lo_off = clamp_big(m.lo) - dq;                      // off >= lo_off <=> d >= lo
     const int up = (kv < Lkv) ? (Lq - 1 - qb) : -1;               // off <= up <=> q < Lq (and the key exists)
