@@ -24,6 +24,9 @@ selects numerics here:
     {"pad_head_dim": bool}  16-bit inputs whose head sizes are not D = Dv in {64, 128} (but at most
                           128) are zero-padded to the next of those so that the fused kernels serve
                           them (default True)
+    {"tile_lists": bool}  False: call the library without tile lists, as a C-ABI caller without a
+                          block mask would; every tile is then visited and the mask evaluated in
+                          each (default True: lists are built from the mask)
 """
 from __future__ import annotations
 
@@ -148,7 +151,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
         flags |= _lib.FLAG_FORCE_GENERIC
     plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, score, flags, opts))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
-    if not mask.is_noop() and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
+    if not mask.is_noop() and opts.get("tile_lists", True) and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
         holder = block_mask if block_mask is not None else _holder_for(mask)
         holder.spec = mask
         for which in (0, 1):

@@ -84,7 +84,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
     part_idx = tl.kv_idx + row * tl.n_kv_blocks;
   } else {
+    // no lists: every tile is visited, and evaluated under a mask that can hide something
     n_full = (p.Lkv + BN - 1) / BN;
+    if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
   }
   // a list entry covers `sub` staged tiles of BN keys (the lists are kListBN-granular);
   // the schedule below runs over (entry, part) pairs flattened into one index
@@ -326,7 +328,9 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       full_idx = tl.full_q_idx + row * tl.n_q_blocks;
       part_idx = tl.q_idx + row * tl.n_q_blocks;
     } else {
+      // no lists: every tile is visited, and evaluated under a mask that can hide something
       n_full = (p.Lq + BM - 1) / BM;
+      if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
     }
     const int nt = n_full + n_part;
     const T* qbase = q + b * p.q_stride[0] + h * p.q_stride[1];

@@ -8,7 +8,7 @@
 // Two kernels.  fwd_mfma_kernel (any supported D, tile lists or not): one workgroup
 // (4 waves) per 128 query rows of one (batch, head), one 32-row block per wave; KV tiles of
 // 64 rows go through two LDS stages (register-prefetched one tile ahead, one workgroup
-// barrier per tile).  fwd_pipe_kernel (D = 64 without tile lists): 256 query rows per
+// barrier per tile).  fwd_pipe_kernel (D = 64, no tile lists, nothing to mask): 256 query rows per
 // workgroup, two blocks per wave, software-pipelined (see there).
 // Per 32-key step and 32-row block:
 //   S^T[kv, q]  = K_step . Q^T          D/16 v_mfma_f32_32x32x16
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
     part_idx = tl.kv_idx + row * tl.n_kv_blocks;
   } else {
+    // no lists: every tile is visited, and evaluated under a mask that can hide something
     n_full = (p.Lkv + BN - 1) / BN;
+    if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
   }
   const int nt = n_full + n_part;
   auto tile_at = [&](int it) -> int {
@@ -332,24 +334,11 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
     for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
   }
 
-  const FlexTileLists& tl = p.tiles;
-  const int32_t* full_idx = nullptr;
-  const int32_t* part_idx = nullptr;
-  int n_full, n_part = 0;
-  if (tl.kv_num) {
-    const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
-    n_full = tl.full_kv_num[row];
-    n_part = tl.kv_num[row];
-    full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
-    part_idx = tl.kv_idx + row * tl.n_kv_blocks;
-  } else {
-    n_full = (p.Lkv + BN - 1) / BN;
-  }
-  const int nt = n_full + n_part;
-  auto tile_at = [&](int it) -> int {
-    if (!full_idx) return it;
-    return it < n_full ? full_idx[it] : part_idx[it - n_full];
-  };
+  // every key tile is visited and nothing is masked: this kernel is launched for problems without tile
+  // lists, with a mask that hides nothing and a key length that is a multiple of the tile (mask code in
+  // the same function costs the unmasked path 3 %)
+  const int nt = p.Lkv / BN;
+  auto tile_at = [&](int it) -> int { return it; };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
@@ -358,7 +347,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
   const int fill_row = lane >> 3;                         // row inside the 8-row group
   auto issue_tile = [&](int stage, int kv0) {
-    const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
+    const int lim = p.Lkv - 1 - kv0;  // guard only: the key length is a multiple of the tile here
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const int r0 = 16 * w + 8 * j;
@@ -406,7 +395,6 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 
   Score2<KIND> sm;
   sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
-  Mask2 visible(p.mask, b, h, p.Lkv);
 
   float16_t oacc[RQ][DB], s_cur;
   float m_run[RQ], l_run[RQ];
@@ -444,19 +432,14 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
 
   const int slot = blockIdx.x >= (gridDim.x >> 1) ? 1 : 0;  // second half of the grid = second workgroup of a compute unit
-  const bool trade = tl.kv_num == nullptr;
   int st = 0;  // LDS stage of the current tile (it % 3)
   for (int it = 0; it < nt; it++) {
     // Two workgroups share a compute unit and the instruction arbiter favours the older wave,
-    // which leaves the younger one behind until it runs alone at the end.  When all workgroups
-    // have the same amount of work (no tile lists), trading the wave priority between them
-    // every tile keeps both advancing at the same pace.  With lists the heavy workgroups are
-    // dispatched first and are the critical path, so the arbiter's preference is kept.
-    if (trade) {
-      if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
-    }
+    // which leaves the younger one behind until it runs alone at the end.  All workgroups have
+    // the same amount of work here, so trading the wave priority between them every tile keeps
+    // both advancing at the same pace.
+    if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
     const int kv0 = t_cur * BN;
-    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
     const int st_n = st == 2 ? 0 : st + 1;
     const T* Ks = Ksm[st];
     const T* Vs = Vsm[st];
@@ -500,17 +483,6 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one matrix instruction
           if (a == 1) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads (V columns)
           __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // six vector instructions
-        }
-        if (masked) {
-          // a real branch whose inputs pass through the asm, so that none of the mask
-          // arithmetic can be hoisted into the unmasked path
-          int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
-          asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-          // most 32x32 blocks of a partial tile are entirely visible or entirely hidden
-          const int cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_opaque - i32),
-                                           __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
-          if (cls == kBlockNone) fill_masked(s_cur);
-          else if (cls == kBlockMixed) mask_block_q(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
         // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
         float m_rel = xhalf_max(block_max(s_cur));
@@ -592,12 +564,12 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 
 template <typename T, int D, int KIND>
 static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
-  // D = 64 without tile lists (every workgroup has the same work): the pipelined kernel with
-  // 256-row workgroups.  With lists the 128-row kernel: twice the workgroups, half the length of the
+  // D = 64 without tile lists or anything to mask (every workgroup has the same work): the pipelined
+  // kernel with 256-row workgroups.  Otherwise the 128-row kernel: twice the workgroups, half the length of the
   // longest one, which is what bounds a causal-like schedule.
   // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
   if constexpr (KIND != FLEX_SCORE_AFFINE) {
-    if (D == 64 && !p.tiles.kv_num) {
+    if (D == 64 && !p.tiles.kv_num && mask_hides_nothing(p.mask) && p.Lkv % kFwdBN == 0) {
       dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
       if (p.flags & FLEX_ROUND_S)
         hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);

@@ -247,6 +247,10 @@ struct Mask2 {
 // bound:  off <= up  &&  (off >= wlo || off <= snk).  Bounds are clamped to
 // +-2^30 so that no subtraction overflows (sequence positions are far smaller).
 // ---------------------------------------------------------------------------
+// a mask that hides nothing: without tile lists every tile then counts as fully visible, otherwise as partial
+__host__ __device__ __forceinline__ bool mask_hides_nothing(const FlexMask& m) {
+  return m.kind == FLEX_MASK_BAND && m.lo == INT32_MIN && m.hi == INT32_MAX;
+}
 constexpr int kBig = 1 << 30;
 __device__ __forceinline__ int clamp_big(int x) { return min(max(x, -kBig), kBig); }
 

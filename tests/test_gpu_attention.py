@@ -494,3 +494,42 @@ def test_bitmap_mask_with_and_without_query_packed_copy(dev):
     wq, wk, wv = ref_attention_bwd(q.cpu(), k.cpu(), v.cpu(), d_o.cpu(), None, mask, strict=True)
     for got, w in zip(grads[0][1:], (wq, wk, wv)):
         assert rel_l2(got.cpu(), w) <= 1e-3
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("kind", ["causal", "window", "bitmap", "none"])
+def test_masks_without_tile_lists(dev, D, kind):
+    """The C ABI allows a call without tile lists: every tile is visited and the mask evaluated in each.  Forward
+    and backward must then give what they give with lists (and the oracle's result)."""
+    print(f"case no tile lists D{D} {kind}", flush=True)
+    B, H, Lq, Lkv = 2, 2, 200, 330
+    g = torch.Generator(device="cpu").manual_seed(11)
+    if kind == "causal":
+        mask, omask = offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq)
+    elif kind == "window":
+        mask, omask = generate_sliding_window(40), o_sliding_window(40)
+    elif kind == "none":
+        mask = omask = None
+    else:
+        keep = torch.rand(1, 1, Lq, Lkv, generator=g) < 0.5
+        keep[..., 0] = True
+        keep_dev = keep.to(dev)
+
+        def mask(b, h, q_idx, kv_idx):
+            t = keep_dev if q_idx.is_cuda else keep
+            return t[0, 0, q_idx.long(), kv_idx.long()]
+        omask = mask
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(torch.float16)
+    q, k, v, d_o = mk(B, H, Lq, D), mk(B, H, Lkv, D), mk(B, H, Lkv, D), mk(B, H, Lq, D)
+    res = []
+    for lists in (True, False):
+        qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+        out = fa.flax_attention_pallas(qd, kd, vd, mask_mod=mask, kernel_options={"tile_lists": lists})
+        out.backward(d_o.to(dev))
+        res.append((out.detach().cpu(), qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()))
+    want = ref_attention(q, k, v, None, omask, strict=True)
+    wq, wk, wv = ref_attention_bwd(q, k, v, d_o, None, omask, strict=True)
+    for name, a, b_, w in zip(("O", "dQ", "dK", "dV"), res[0], res[1], (want, wq, wk, wv)):
+        print(f"  {name}: lists vs none {max_abs(a, b_):.3e}; none vs oracle rel-L2 {rel_l2(b_, w):.3e}", flush=True)
+        assert rel_l2(b_, w) <= 1e-3 and max_abs(b_, w) <= 2e-2 * max(1.0, w.abs().max().item())
+        assert max_abs(a, b_) <= 4e-3 * max(1.0, w.abs().max().item())
