@@ -1,0 +1,108 @@
+"""The C ABI called directly (ctypes, raw pointers), for the promises of include/flexattn.h that the Python layer
+never exercises by itself: optional pointers, calls without tile lists, error returns that launch nothing."""
+import ctypes as C
+import math
+
+import pytest
+import torch
+
+from flaxattention_amd import _lib
+from oracle import max_abs, o_causal_mask, ref_attention, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+INT_MIN, INT_MAX = -2 ** 31, 2 ** 31 - 1
+
+
+def _params(q, k, v, o, lo=INT_MIN, hi=INT_MAX):
+    B, H, Lq, D = q.shape
+    p = _lib.FlexAttnParams()
+    p.dtype = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[q.dtype]
+    p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = B, H, k.shape[1], Lq, k.shape[2], D, v.shape[3]
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
+        getattr(p, name)[:] = [t.stride(0), t.stride(1), t.stride(2)]
+    p.scale, p.flags = 1.0 / math.sqrt(D), 1   # FLEX_ROUND_S
+    p.score.kind = 0
+    p.mask.kind, p.mask.lo, p.mask.hi, p.mask.sink = 0, lo, hi, -1
+    return p
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _inputs(dev, B, H, Lq, Lkv, D, dtype=torch.float16):
+    g = torch.Generator(device="cpu").manual_seed(7)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(dtype).to(dev)
+    return mk(B, H, Lq, D), mk(B, H, Lkv, D), mk(B, H, Lkv, D)
+
+
+def test_forward_without_lse_and_without_lists(dev):
+    print("case C ABI forward, causal band mask, no lists, lse2 NULL", flush=True)
+    L = _lib.lib()
+    q, k, v = _inputs(dev, 2, 2, 256, 256, 64)
+    o1, o2 = torch.empty_like(q), torch.empty_like(q)
+    lse = torch.empty(2, 2, 256, dtype=torch.float32, device=dev)
+    p = _params(q, k, v, o1, lo=0)   # d = q - kv >= 0: causal
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o1.data_ptr(), lse.data_ptr(), None, _stream()) == 0
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o2.data_ptr(), None, None, _stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
+    want, want_lse = ref_attention(q.cpu(), k.cpu(), v.cpu(), None, o_causal_mask, strict=True, return_lse=True)
+    assert rel_l2(o1.cpu(), want) <= 1e-3 and max_abs(lse.cpu() * math.log(2.0), want_lse) <= 2e-2
+
+
+def test_errors_launch_nothing(dev):
+    print("case C ABI error returns", flush=True)
+    L = _lib.lib()
+    q, k, v = _inputs(dev, 1, 2, 128, 128, 64)
+    o = torch.full_like(q, 7.0)
+    p = _params(q, k, v, o)
+    assert L.flexattn_fwd(p, None, k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
+    assert b"null" in L.flexattn_last_error()
+    p.Lkv = 0
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
+    assert b"non-positive" in L.flexattn_last_error()
+    p = _params(q, k, v, o)
+    p.Hkv = 3   # 2 query heads do not divide over 3 KV heads
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
+    p = _params(q, k, v, o)
+    p.q_index_base = 64
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
+    p = _params(q, k, v, o)   # decode takes at most 64 query columns
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    assert L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, 2, ws.data_ptr(), _stream()) != 0
+    assert b"Lq <= 64" in L.flexattn_last_error()
+    p.mask.kind = 1   # a bitmap mask without a bitmap
+    assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
+    torch.cuda.synchronize()
+    assert bool((o == 7.0).all())   # nothing was launched by any of the refused calls
+
+
+def test_block_mask_build_with_optional_outputs(dev):
+    print("case C ABI block-mask build, some outputs NULL", flush=True)
+    L = _lib.lib()
+    B, H, nq, nkv = 2, 3, 5, 7
+    m = _lib.FlexMask()
+    m.kind, m.lo, m.hi, m.sink = 0, 0, 200, 3   # causal window of 200 with 4 sink keys
+    i32 = dict(dtype=torch.int32, device=dev)
+    full = {n: torch.empty(s, **i32) for n, s in (("kv_num", (B, H, nq)), ("kv_idx", (B, H, nq, nkv)),
+                                                  ("full_kv_num", (B, H, nq)), ("full_kv_idx", (B, H, nq, nkv)),
+                                                  ("q_num", (B, H, nkv)), ("q_idx", (B, H, nkv, nq)),
+                                                  ("full_q_num", (B, H, nkv)), ("full_q_idx", (B, H, nkv, nq)))}
+    ws = torch.empty(L.flexattn_block_mask_workspace_bytes(B, H, nq, nkv), dtype=torch.uint8, device=dev)
+    ptr = lambda t: t.data_ptr()
+    order = ("kv_num", "kv_idx", "full_kv_num", "full_kv_idx", "q_num", "q_idx", "full_q_num", "full_q_idx")
+    assert L.flexattn_block_mask_build(C.byref(m), B, H, nq, nkv, 128, 128, *[ptr(full[n]) for n in order],
+                                       ws.data_ptr(), _stream()) == 0
+    only = {n: torch.full_like(full[n], -5) for n in ("kv_num", "full_q_idx")}
+    assert L.flexattn_block_mask_build(C.byref(m), B, H, nq, nkv, 128, 128,
+                                       *[ptr(only[n]) if n in only else None for n in order],
+                                       ws.data_ptr(), _stream()) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(only["kv_num"], full["kv_num"]) and torch.equal(only["full_q_idx"], full["full_q_idx"])
+    # the transposed counts agree with the row counts: same number of partial / full tiles either way
+    assert int(full["kv_num"].sum()) == int(full["q_num"].sum())
+    assert int(full["full_kv_num"].sum()) == int(full["full_q_num"].sum())
+    assert L.flexattn_block_mask_build(C.byref(m), B, H, 0, nkv, 128, 128, *[None] * 8, ws.data_ptr(), _stream()) != 0
+    assert L.flexattn_block_mask_build(C.byref(m), B, H, nq, nkv, 128, 128, *[None] * 8, None, _stream()) != 0
