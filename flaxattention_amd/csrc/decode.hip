@@ -71,12 +71,14 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   }
   if (kQInLds) __syncthreads();
 
-  // schedule: list entries (64-row tiles of query block 0) when given and G == 1, else every step
+  // schedule: list entries (64-key tiles of the query block the rows sit in) when given at that
+  // granularity, with all rows in one query block, and G == 1; else every step with the mask
+  // evaluated in each
   const FlexTileLists& tl = p.tiles;
   const int32_t* full_idx = nullptr;
   const int32_t* part_idx = nullptr;
   int n_full = 0, steps_total;
-  if (tl.kv_num && G == 1) {
+  if (tl.kv_num && G == 1 && tl.kv_block == 2 * kStep && p.q_index_base % tl.q_block + p.Lq <= tl.q_block) {
     const int64_t row = (b * tl.stride_b + hk * tl.stride_h) * tl.n_q_blocks + p.q_index_base / tl.q_block;
     n_full = tl.full_kv_num[row];
     const int n_part = tl.kv_num[row];
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     if (!full_idx) return st * kStep;
     const int item = st >> 1;
     const int tile = item < n_full ? full_idx[item] : part_idx[item - n_full];
-    return tile * 64 + (st & 1) * kStep;
+    return tile * (2 * kStep) + (st & 1) * kStep;
   };
   const int per = (steps_total + splits - 1) / splits;
   const int st_begin = split * per, st_end = min(st_begin + per, steps_total);

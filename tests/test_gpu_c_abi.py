@@ -106,3 +106,36 @@ def test_block_mask_build_with_optional_outputs(dev):
     assert int(full["full_kv_num"].sum()) == int(full["full_q_num"].sum())
     assert L.flexattn_block_mask_build(C.byref(m), B, H, 0, nkv, 128, 128, *[None] * 8, ws.data_ptr(), _stream()) != 0
     assert L.flexattn_block_mask_build(C.byref(m), B, H, nq, nkv, 128, 128, *[None] * 8, None, _stream()) != 0
+
+
+def test_decode_with_lists_of_another_granularity(dev):
+    """Tile lists built at 128 x 128 (the API's block size) instead of the 128 x 64 the decode kernel walks: the
+    kernel must not read them as 64-key tiles.  Result = the call without lists."""
+    print("case C ABI decode, lists at 128 x 128", flush=True)
+    import flaxattention_amd as fa
+    from flaxattention_amd.core.blockmask import build_lists
+    from flaxattention_amd.masks import generate_sliding_window
+    L = _lib.lib()
+    B, H, Lq, Lkv, D = 2, 4, 16, 1024, 64
+    q, k, v = _inputs(dev, B, H, Lq, Lkv, D)
+    outs = []
+    spec = generate_sliding_window(300)
+    spec_off = type(spec)(lo=spec.lo, hi=spec.hi, sink=spec.sink, q_offset=Lkv - Lq)
+    lists = build_lists(spec_off, 1, 1, 1, Lkv // 128, 128, 128, dev)
+    for use_lists in (False, True):
+        o = torch.empty_like(q)
+        p = _params(q, k, v, o, lo=spec.lo, hi=spec.hi)
+        p.mask.q_offset = Lkv - Lq
+        if use_lists:
+            t = p.tiles
+            t.kv_num, t.kv_idx = lists["kv_num_blocks"].data_ptr(), lists["kv_indices"].data_ptr()
+            t.full_kv_num, t.full_kv_idx = lists["full_kv_num_blocks"].data_ptr(), lists["full_kv_indices"].data_ptr()
+            t.q_block, t.kv_block, t.n_q_blocks, t.n_kv_blocks = 128, 128, 1, Lkv // 128
+        ws = torch.empty(L.flexattn_decode_workspace_bytes(p, 4), dtype=torch.uint8, device=dev)
+        assert L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, 4, ws.data_ptr(), _stream()) == 0
+        torch.cuda.synchronize()
+        outs.append(o)
+    assert torch.equal(outs[0], outs[1])
+    want = fa.flax_attention(q, k, v, block_mask=fa.create_block_mask(spec_off, 1, 1, Lq, Lkv, device=dev),
+                             kernel_options={"decode": False})
+    assert max_abs(outs[0].cpu(), want.cpu()) <= 4e-3
