@@ -306,7 +306,13 @@ def _nothing_to_attend(query: Array, key: Array) -> bool:
 
 
 def _as_kernel_layout(t: Array) -> Array:
-    return t if t.stride(-1) == 1 else t.contiguous()
+    """The kernels read 16-byte chunks along a contiguous feature axis: anything else (a transposed feature axis, a
+    view that starts in the middle of a row) is copied once."""
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    if t.data_ptr() % 16 != 0 or (not t.is_contiguous() and any(s % 8 != 0 for s in t.stride()[:-1])):
+        t = t.clone(memory_format=torch.contiguous_format)
+    return t
 
 
 def _pad_head_dims(q: Array, k: Array, v: Array, kernel_options) -> Tuple[Array, Array, Array]:

@@ -533,3 +533,19 @@ def test_masks_without_tile_lists(dev, D, kind):
         print(f"  {name}: lists vs none {max_abs(a, b_):.3e}; none vs oracle rel-L2 {rel_l2(b_, w):.3e}", flush=True)
         assert rel_l2(b_, w) <= 1e-3 and max_abs(b_, w) <= 2e-2 * max(1.0, w.abs().max().item())
         assert max_abs(a, b_) <= 4e-3 * max(1.0, w.abs().max().item())
+
+
+def test_views_that_start_inside_a_row(dev):
+    """Inputs sliced along the feature axis (not 16-byte aligned, row stride not a multiple of 8 elements for one of
+    them) are copied once by the front-end instead of being refused by the fused kernels."""
+    print("case misaligned views", flush=True)
+    g = torch.Generator(device="cpu").manual_seed(2)
+    big = torch.randn(3, 2, 2, 150, 72, generator=g).to(torch.float16).to(dev)
+    q, k, v = big[0, ..., 4:68], big[1, ..., 4:68], big[2, ..., 8:72]
+    assert q.data_ptr() % 16 != 0 and q.stride(-1) == 1
+    out = fa.flax_attention(q, k, v)
+    want = fa.flax_attention(q.contiguous(), k.contiguous(), v.contiguous())
+    assert torch.equal(out, want)
+    odd = torch.randn(2, 2, 150, 68, generator=g).to(torch.float16).to(dev)[..., :64]   # row stride 68
+    out = fa.flax_attention(odd, k, v)
+    assert torch.equal(out, fa.flax_attention(odd.contiguous(), k.contiguous(), v.contiguous()))
