@@ -24,7 +24,9 @@ constexpr int kBM = 128;     // query tile (list granularity)
 constexpr int kBN = 128;     // key tile staged per step by the dQ kernel at D = 64 (half of it at D = 128)
 constexpr int kListBN = 128; // key granularity of the backward tile lists = key rows of a dK/dV workgroup
 
-template <typename T, int D, int KIND, bool ROUND_S>
+// MASKED = false: the caller guarantees that there is nothing to mask (no tile lists, a mask that hides nothing,
+// key length a multiple of the tile); that instantiation carries no mask code, which is worth 2 % on its own.
+template <typename T, int D, int KIND, bool ROUND_S, bool MASKED>
 __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   const float neg_delta = -delta;
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
-    const bool masked = (it >= n_full_t) || (kv0 + BN > p.Lkv);
+    const bool masked = MASKED && ((it >= n_full_t) || (kv0 + BN > p.Lkv));
     const T* Ks = Ksm[it & 1];
     const T* Vs = Vsm[it & 1];
     if (it + 1 < nt) {
@@ -548,18 +550,29 @@ static int launch_dkv(const FlexAttnParams& p, const void* q, const void* k, con
 }
 
 template <typename T, int D, int KIND, bool RS>
+static void launch_dq(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                      const void* d_o, void* dq, float* delta, hipStream_t s) {
+  const int nqt = (p.Lq + kBM - 1) / kBM;
+  constexpr int BN = D == 64 ? kBN : kBN / 2;   // the kernel's key tile
+  const dim3 grid(nqt * p.Hq * p.B);
+  if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0)
+    hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v,
+                       (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+  else
+    hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v,
+                       (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+}
+
+template <typename T, int D, int KIND, bool RS>
 static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  const int nqt = (p.Lq + kBM - 1) / kBM;
   if (!(p.flags & FLEX_BWD_ONLY_DKV)) {
     if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.p0 > 0.f && p.score.p1 > 0.f) {
       // positive factors: the derivative folds into the exponent
       constexpr int KF = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardFold : KIND;
-      hipLaunchKernelGGL((bwd_dq_kernel<T, D, KF, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
-                         (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+      launch_dq<T, D, KF, RS>(p, q, k, v, o, lse2, d_o, dq, delta, s);
     } else {
-      hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS>), dim3(nqt * p.Hq * p.B), dim3(256), 0, s, p, (const T*)q, (const T*)k,
-                         (const T*)v, (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
+      launch_dq<T, D, KIND, RS>(p, q, k, v, o, lse2, d_o, dq, delta, s);
     }
   }
   if (p.flags & FLEX_BWD_ONLY_DQ) return 0;
