@@ -279,7 +279,11 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int BM = kBM, BN = kListBN;
   constexpr int kDkvThreads = DkvShape<D>::kThreads, QBW = DkvShape<D>::kQBlocks;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
+  // D = 64: the Q and dO tiles land in LDS straight from global memory (unpadded rows, chunk c of row r at
+  // position c ^ lds_swz(r): conflict-free for the row-fragment and the transposing reads); D = 128 stages them
+  // through registers into padded rows
+  constexpr bool DIRECT = D == 64;
+  constexpr int DS = D / 16, DB = D / 32, ROWE = DIRECT ? D : D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
   // LDS stages of (Q tile, dO tile, lse, -delta).  D = 64 keeps two, so that one workgroup
   // barrier per tile suffices; with D = 128 a second stage would cost the second workgroup
   // of the compute unit, so one stage is refilled between two barriers.
@@ -312,6 +316,21 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
   for (int db = 0; db < DB; db++)
 #pragma unroll
     for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
+  // element offsets inside a 32-row block of a tile: row fragments (row i32, chunk 2s + g) and transposing
+  // reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
+  const int kz = DIRECT ? (g ^ lds_swz<D>(i32)) : g;
+  int toff[2][DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
+#pragma unroll
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        const int pos = DIRECT ? (chunk ^ lds_swz<D>(rl + 8 * e)) : chunk;
+        toff[e][db] = (rl + 8 * e) * ROWE + pos * 8 + 4 * (i16 & 1);
+      }
+  }
 
   const FlexTileLists& tl = p.tiles_bwd;
   Score2<KIND> sm;
@@ -343,14 +362,35 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       if (!full_idx) return it;
       return it < n_full ? full_idx[it] : part_idx[it - n_full];
     };
-    u32x4 qreg[NLD], oreg[NLD];
+    u32x4 qreg[DIRECT ? 1 : NLD], oreg[DIRECT ? 1 : NLD];
     float lreg = INFINITY, dreg = 0.f;
-    auto load_tile = [&](int q0) {
+    // direct fetch: wave w fills rows [32w, 32w + 32) of the Q and the dO tile, 8 rows per instruction; the lane
+    // that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
+    auto issue_tile = [&](int st, int q0) {
+      T* Qw = stage_q(st);
+      T* Ow = Qw + BM * ROWE;
+      const int lim = p.Lq - 1 - q0;  // rows past the end: clamped (finite filler; their lse is +inf, so P = 0)
 #pragma unroll
-      for (int j = 0; j < NLD; j++) {
-        const int c = tid + kDkvThreads * j, r = min(c / CPR, p.Lq - 1 - q0), cc = c % CPR;  // clamped: finite filler
-        qreg[j] = *reinterpret_cast<const u32x4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
-        oreg[j] = *reinterpret_cast<const u32x4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
+      for (int j = 0; j < 4; j++) {
+        const int r0 = 32 * w + 8 * j;
+        const int chunk = (lane & 7) ^ lds_swz<D>(8 * j + (lane >> 3));  // the wave's first row is a multiple of 16
+        const int row = min(r0 + (lane >> 3), lim);
+        const T* qg = qbase + (int64_t)(q0 + row) * p.q_stride[2] + chunk * 8;
+        const T* og = dobase + (int64_t)(q0 + row) * D + chunk * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)qg,
+                                         (__attribute__((address_space(3))) void*)(Qw + r0 * ROWE), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)og,
+                                         (__attribute__((address_space(3))) void*)(Ow + r0 * ROWE), 16, 0, 0);
+      }
+    };
+    auto load_tile = [&](int q0) {
+      if constexpr (!DIRECT) {
+#pragma unroll
+        for (int j = 0; j < NLD; j++) {
+          const int c = tid + kDkvThreads * j, r = min(c / CPR, p.Lq - 1 - q0), cc = c % CPR;  // clamped: finite filler
+          qreg[j] = *reinterpret_cast<const u32x4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
+          oreg[j] = *reinterpret_cast<const u32x4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
+        }
       }
       lreg = INFINITY;
       dreg = 0.f;
@@ -366,11 +406,13 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       T* Qw = stage_q(st);
       T* Ow = Qw + BM * ROWE;
       float* lw = reinterpret_cast<float*>(Ow + BM * ROWE);
+      if constexpr (!DIRECT) {
 #pragma unroll
-      for (int j = 0; j < NLD; j++) {
-        const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
-        *reinterpret_cast<u32x4*>(Qw + r * ROWE + cc * 8) = qreg[j];
-        *reinterpret_cast<u32x4*>(Ow + r * ROWE + cc * 8) = oreg[j];
+        for (int j = 0; j < NLD; j++) {
+          const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
+          *reinterpret_cast<u32x4*>(Qw + r * ROWE + cc * 8) = qreg[j];
+          *reinterpret_cast<u32x4*>(Ow + r * ROWE + cc * 8) = oreg[j];
+        }
       }
       if (tid < BM) {
         lw[tid] = lreg;        // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
@@ -378,10 +420,14 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       }
     };
     __syncthreads();  // the stages may still be in use by the previous head of the group
-    if (nt > 0) load_tile(t_cur * BM);
+    if (nt > 0) {
+      if constexpr (DIRECT) issue_tile(0, t_cur * BM);
+      load_tile(t_cur * BM);
+    }
     if (NSTG == 2) {
       if (nt > 0) store_tile(0);
       if (nt > 1) load_tile(t_nxt * BM);
+      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
     }
     for (int it = 0; it < nt; it++) {
@@ -394,8 +440,11 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       const float* del_s = lse_s + BM;
       if (NSTG == 2) {
         if (it + 1 < nt) {
-          // the other stage was last read before the previous barrier: refill it with the
-          // tile prefetched into registers, then start fetching the one after
+          // the other stage was last read before the previous barrier: refill it (D = 64: the
+          // tile itself is fetched straight into it now and awaited at the end of this tile; lse
+          // and delta, like whole tiles at D = 128, were prefetched into registers), then start
+          // fetching the one after
+          if constexpr (DIRECT) issue_tile((it + 1) & 1, t_nxt * BM);
           store_tile((it + 1) & 1);
           t_cur = t_nxt;
           if (it + 2 < nt) {
@@ -435,12 +484,12 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
         for (int e = 0; e < 4; e++) { sacc[4 * rr + e] = 0.f; dpacc[4 * rr + e] = d4[e]; }
       }
       {
-        const T* qp = Qs + (qrow_w + i32) * ROWE + 8 * g;
-        const T* op = Os + (qrow_w + i32) * ROWE + 8 * g;
+        const T* qp = Qs + (qrow_w + i32) * ROWE;
+        const T* op = Os + (qrow_w + i32) * ROWE;
 #pragma unroll
         for (int s = 0; s < DS; s++) {
-          sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + 16 * s), kf[s], sacc);
-          dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + 16 * s), vf[s], dpacc);
+          sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + (((2 * s) ^ kz) * 8)), kf[s], sacc);
+          dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + (((2 * s) ^ kz) * 8)), vf[s], dpacc);
         }
       }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
@@ -489,14 +538,15 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const int off = (qrow_w + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-          vec8 a_do = join8<vec8>(lds_read_tr(Os + off), lds_read_tr(Os + off + 8 * ROWE));
+          const int base = (qrow_w + 16 * tt) * ROWE;
+          vec8 a_do = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
           dvacc[db] = Frag<T>::mfma(a_do, pf[tt], dvacc[db]);
-          vec8 a_q = join8<vec8>(lds_read_tr(Qs + off), lds_read_tr(Qs + off + 8 * ROWE));
+          vec8 a_q = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
           dkacc[db] = Frag<T>::mfma(a_q, dsf[tt], dkacc[db]);
         }
       }
       }  // query blocks of this wave
+      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed
       __syncthreads();
     }
   }
@@ -523,7 +573,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 }
 
 template <int D, typename T> constexpr size_t dkv_smem() {
-  return DkvShape<D>::kStages * ((size_t)2 * kBM * (D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
+  return DkvShape<D>::kStages * ((size_t)2 * kBM * (D == 64 ? D : D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
 }
 
 template <typename T, int D, int KIND, bool RS, bool BITS>
