@@ -492,6 +492,19 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
           dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + (((2 * s) ^ kz) * 8)), vf[s], dpacc);
         }
       }
+      // D = 64 has the registers to fetch the transposed dO and Q fragments of the closing products now, under the
+      // softmax arithmetic, instead of right before their use (1.7 % of the kernel's time)
+      vec8 a_do[2][DB], a_q[2][DB];
+      if constexpr (DIRECT) {
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) {
+            const int base = (qrow_w + 16 * tt) * ROWE;
+            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
+            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
+          }
+      }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
       float16_t gacc;
       if constexpr (KIND == kScoreCheckerboardKv) key_grad = sm.key_grad;
@@ -539,10 +552,12 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 #pragma unroll
         for (int db = 0; db < DB; db++) {
           const int base = (qrow_w + 16 * tt) * ROWE;
-          vec8 a_do = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
-          dvacc[db] = Frag<T>::mfma(a_do, pf[tt], dvacc[db]);
-          vec8 a_q = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
-          dkacc[db] = Frag<T>::mfma(a_q, dsf[tt], dkacc[db]);
+          if constexpr (!DIRECT) {
+            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
+            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
+          }
+          dvacc[db] = Frag<T>::mfma(a_do[tt][db], pf[tt], dvacc[db]);
+          dkacc[db] = Frag<T>::mfma(a_q[tt][db], dsf[tt], dkacc[db]);
         }
       }
       }  // query blocks of this wave
