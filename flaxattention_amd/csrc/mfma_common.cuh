@@ -186,11 +186,15 @@ template <> struct Score2<FLEX_SCORE_TANH_SOFTCAP> {
   __device__ __forceinline__ void tile(int q, int kvb) {}
   __device__ __forceinline__ void tileT(int qb, int kv) {}
   __device__ __forceinline__ float tanh_(float s) const {
-    float t = fast_exp2(fminf(s * a, 60.f));
+    // no clamp: for a large argument v_exp_f32 gives +inf, v_rcp_f32 of that 0, and the result is exactly 1
+    float t = fast_exp2(s * a);
     return 1.f - 2.f * fast_rcp(t + 1.f);
   }
-  __device__ __forceinline__ float apply(float s, int off) const { return cap2 * tanh_(s); }
-  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(cap2, tanh_(s), -m); }
+  // r = 1 / (2^(a s) + 1), tanh = 1 - 2 r: cap2 * tanh - m = (cap2 - m) - 2 cap2 r, one fused multiply-add per entry
+  // (cap2 - m is common to the entries of a block)
+  __device__ __forceinline__ float half_gap(float s) const { return fast_rcp(fast_exp2(s * a) + 1.f); }
+  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(-2.f * cap2, half_gap(s), cap2); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const { return fmaf(-2.f * cap2, half_gap(s), cap2 - m); }
   __device__ __forceinline__ float grad(float s, int off) const { float t = tanh_(s); return 1.f - t * t; }
 };
 

@@ -549,3 +549,24 @@ def test_views_that_start_inside_a_row(dev):
     odd = torch.randn(2, 2, 150, 68, generator=g).to(torch.float16).to(dev)[..., :64]   # row stride 68
     out = fa.flax_attention(odd, k, v)
     assert torch.equal(out, fa.flax_attention(odd.contiguous(), k.contiguous(), v.contiguous()))
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_softcap_saturates_cleanly(dev, D):
+    """Scores far beyond the cap (|s| / cap in the hundreds): tanh is exactly +-1 there, its derivative 0, and nothing
+    turns into NaN in the fused kernels (their tanh goes through exp2 and a reciprocal without a clamp)."""
+    print(f"case soft-cap saturation D{D}", flush=True)
+    B, H, L = 1, 2, 192
+    g = torch.Generator(device="cpu").manual_seed(4)
+    mk = lambda *s: (6.0 * torch.randn(*s, generator=g, dtype=torch.float32)).to(torch.float16)
+    q, k, v, d_o = mk(B, H, L, D), mk(B, H, L, D), mk(B, H, L, D) / 6, mk(B, H, L, D) / 6
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    out = fa.flax_attention(qd, kd, vd, score_mod=generate_tanh_softcap(2.0))
+    out.backward(d_o.to(dev))
+    for t in (out, qd.grad, kd.grad, vd.grad):
+        assert bool(torch.isfinite(t).all())
+    want = ref_attention(q, k, v, o_tanh_softcap(2.0), None, strict=True)
+    wq, wk, wv = ref_attention_bwd(q, k, v, d_o, o_tanh_softcap(2.0), None, strict=True)
+    assert rel_l2(out.detach().cpu(), want) <= 1e-3
+    for got, w in ((qd.grad, wq), (kd.grad, wk), (vd.grad, wv)):
+        assert rel_l2(got.cpu(), w) <= 2e-3 and max_abs(got.cpu(), w) <= 2e-2 * max(1.0, w.abs().max().item())
