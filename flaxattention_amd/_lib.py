@@ -67,6 +67,7 @@ EXPORTS = [
     "flexattn_decode_workspace_bytes", "flexattn_decode",
     "flexattn_probe_mfma",
     "flexattn_probe_mix",
+    "flexattn_probe_read",
 ]
 
 _lib: Optional[C.CDLL] = None
@@ -113,6 +114,7 @@ def lib() -> C.CDLL:
     L.flexattn_decode.argtypes = [C.POINTER(FlexAttnParams)] + [C.c_void_p] * 5 + [C.c_int32, C.c_void_p, C.c_void_p]
     L.flexattn_probe_mfma.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
     L.flexattn_probe_mix.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
+    L.flexattn_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     _lib = L
     return L
 

@@ -93,6 +93,35 @@ __global__ __launch_bounds__(256, 2) void mix_probe_kernel(float* __restrict__ s
 
 void flex_set_error(const char* fmt, ...);
 
+namespace flex {
+// A streaming read and nothing else: every thread folds 16-byte loads (four independent ones per trip) into a value
+// that is practically never written.
+__global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict__ src, size_t n_vec, float* __restrict__ sink) {
+  const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x, total = (size_t)gridDim.x * blockDim.x;
+  uint4 acc = make_uint4(0, 0, 0, 0);
+  for (size_t i = tid; i < n_vec; i += 4 * total) {
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    const uint4 a = src[i], b = i + total < n_vec ? src[i + total] : z;
+    const uint4 c = i + 2 * total < n_vec ? src[i + 2 * total] : z, d = i + 3 * total < n_vec ? src[i + 3 * total] : z;
+    acc.x ^= a.x ^ b.x ^ c.x ^ d.x; acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
+    acc.z ^= a.z ^ b.z ^ c.z ^ d.z; acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[tid & 0xffff] = 1.f;
+}
+}  // namespace flex
+
+// 1024 workgroups of 256 threads (the grid a bare read is fastest with here) over `bytes` of device memory.
+extern "C" int flexattn_probe_read(const void* src, size_t bytes, float* sink, void* stream) {
+  if (!src || !sink || bytes < 16 || ((uintptr_t)src & 15)) {
+    flex_set_error("flexattn_probe_read: needs a 16-byte aligned device buffer of at least 16 bytes and a sink of 65536 floats");
+    return 1;
+  }
+  hipLaunchKernelGGL(flex::read_probe_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, (const uint4*)src, bytes / 16, sink);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { flex_set_error("flexattn_probe_read: launch failed: %s", hipGetErrorString(e)); return 2; }
+  return 0;
+}
+
 // 512 workgroups of 4 waves (two waves per SIMD on 256 compute units), 8 * iters MFMAs per wave.
 extern "C" int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, void* stream) {
   if (!sink || iters <= 0) { flex_set_error("flexattn_probe_mfma: needs a device buffer of 512*256 floats and iters > 0"); return 1; }

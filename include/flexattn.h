@@ -215,6 +215,11 @@ int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, fl
 int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch,
                        flexattn_stream_t stream);
 
+/* Third measurement aid without counterpart in the reference: a kernel that only reads `bytes` of device memory
+ * (16-byte loads, 1024 workgroups), for the read rate that memory delivers to a kernel that does nothing else; the
+ * decode kernel is held against it.  `sink`: 65536 floats, practically never written. */
+int flexattn_probe_read(const void* src, size_t bytes, float* sink, flexattn_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -88,6 +88,13 @@ def test_mfma_probe_runs(dev):
         assert flops.value == 512 * 4 * nm * 3 * 2 * 32 * 32 * 16
         assert torch.isfinite(sink).all()
     assert L.flexattn_probe_mix(sink.data_ptr(), 3, 7, None, None) != 0 and b"probe_mix" in L.flexattn_last_error()
+    # the read probe reads its buffer and (practically never) writes the sink
+    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
+    small = torch.zeros(65536, dtype=torch.float32, device=dev)
+    assert L.flexattn_probe_read(src.data_ptr(), src.numel(), small.data_ptr(), torch.cuda.current_stream(dev).cuda_stream) == 0
+    torch.cuda.synchronize()
+    assert float(small.sum()) <= 1.0
+    assert L.flexattn_probe_read(None, 1 << 20, small.data_ptr(), None) != 0 and b"probe_read" in L.flexattn_last_error()
 
 
 def test_decode_is_chosen_automatically(dev):
