@@ -26,7 +26,9 @@ constexpr int kFwdBN = 64;
 constexpr int kFwdBM = 128;   // query rows of a list-driven workgroup = q granularity of the forward lists
 constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dense kernel (D = 64, no lists)
 
-template <typename T, int D, int KIND, bool ROUND_S>
+// BITS: the mask is a bitmap.  Band masks get an instantiation of their own, without the bitmap code and the scalar
+// registers its pointers and strides occupy.
+template <typename T, int D, int KIND, bool ROUND_S, bool BITS>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2) {
@@ -111,7 +113,6 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 
   Score2<KIND> sm;
   sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
-  Mask2 visible(p.mask, b, h, p.Lkv);
 
   float16_t oacc[RQ][DB];
   float m_run[RQ], l_run[RQ];
@@ -149,7 +150,14 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
       // entirely hidden (the step is skipped)
       int cls = kBlockAll;
-      if (masked) cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+      if (masked) {
+        if constexpr (BITS) {
+          const Mask2 visible(p.mask, b, h, p.Lkv);
+          cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        } else {
+          cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        }
+      }
       if (cls != kBlockNone) {
       sm.tile(q_row0, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
       // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
@@ -199,7 +207,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
           // none of it can be hoisted into the unmasked path (it costs as much as the softmax)
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-          mask_block_q(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+          const Mask2 visible(p.mask, b, h, p.Lkv);
+          mask_block_q<BITS>(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
       }
       // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
@@ -579,10 +588,14 @@ static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, con
     }
   }
   dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B);
-  if (p.flags & FLEX_ROUND_S)
-    hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
-  else
-    hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+  const bool bits = p.mask.kind == FLEX_MASK_BITS;
+  if (p.flags & FLEX_ROUND_S) {
+    if (bits) hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+    else hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, true, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+  } else {
+    if (bits) hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, false, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+    else hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, false, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+  }
 }
 
 template <typename T, int D>

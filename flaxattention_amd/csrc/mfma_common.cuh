@@ -290,10 +290,12 @@ __device__ __forceinline__ void fill_masked(float16_t& x) {
 }
 
 // one 32-key block: register r holds key kv0 + 4*g + acc_row(r); lane owns query q
+// BITS = false: the caller knows that the mask is a band mask.
+template <bool BITS = true>
 __device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
                                              int Lkv) {
   const int kvb = kv0 + 4 * g;
-  if (m.kind == FLEX_MASK_BAND) {
+  if (!BITS || m.kind == FLEX_MASK_BAND) {
     const int dq = q + m.q_offset - kvb;                           // d at off = 0; d = dq - off
     const int up = min(dq - clamp_big(m.lo), Lkv - 1 - kvb);       // off <= up  <=>  d >= lo && kv < Lkv
     if (m.hi >= kBig) {
