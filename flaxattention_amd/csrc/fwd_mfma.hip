@@ -153,7 +153,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       if (masked) {
         if constexpr (BITS) {
           const Mask2 visible(p.mask, b, h, p.Lkv);
-          cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+          cls = block_class<true>(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
         } else {
           cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
         }
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
           int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
           asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
           const Mask2 visible(p.mask, b, h, p.Lkv);
-          mask_block_q<BITS>(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+          mask_block_q<BITS, BITS>(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
       }
       // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----

@@ -275,9 +275,11 @@ __device__ __forceinline__ int band_block_class(const FlexMask& m, int q_first, 
 // The same for any mask: a bitmap answers from its table of block classes when it carries one.
 // q_first and kv_first are multiples of 32.  The table describes the padded index range, so a
 // block that reaches past the real lengths is never reported as entirely visible.
+// KNOWN_BITS: the caller knows that the mask is a bitmap (no band arithmetic is compiled in).
+template <bool KNOWN_BITS = false>
 __device__ __forceinline__ int block_class(const FlexMask& m, const Mask2& visible, int q_first, int kv_first, int Lq,
                                            int Lkv) {
-  if (m.kind == FLEX_MASK_BAND) return band_block_class(m, q_first, kv_first, Lq, Lkv);
+  if (!KNOWN_BITS && m.kind == FLEX_MASK_BAND) return band_block_class(m, q_first, kv_first, Lq, Lkv);
   if (!visible.ev.blk_bh) return kBlockMixed;
   if (kv_first >= Lkv || q_first >= Lq) return kBlockNone;
   const int c = visible.ev.blk_bh[(int64_t)(q_first >> 5) * visible.ev.blk_stride_q + (kv_first >> 5)];
@@ -291,11 +293,11 @@ __device__ __forceinline__ void fill_masked(float16_t& x) {
 
 // one 32-key block: register r holds key kv0 + 4*g + acc_row(r); lane owns query q
 // BITS = false: the caller knows that the mask is a band mask.
-template <bool BITS = true>
+template <bool BITS = true, bool KNOWN_BITS = false>
 __device__ __forceinline__ void mask_block_q(float16_t& x, const FlexMask& m, const Mask2& visible, int q, int kv0, int g,
                                              int Lkv) {
   const int kvb = kv0 + 4 * g;
-  if (!BITS || m.kind == FLEX_MASK_BAND) {
+  if (!KNOWN_BITS && (!BITS || m.kind == FLEX_MASK_BAND)) {
     const int dq = q + m.q_offset - kvb;                           // d at off = 0; d = dq - off
     const int up = min(dq - clamp_big(m.lo), Lkv - 1 - kvb);       // off <= up  <=>  d >= lo && kv < Lkv
     if (m.hi >= kBig) {
@@ -331,10 +333,10 @@ __device__ __forceinline__ void mask_tile_q(float16_t (&x)[2], const FlexMask& m
 
 // Lane owns key kv; register r holds query qb + acc_row(r) (qb already includes 4*g).
 // BITS = false: the caller knows that the mask is a band mask.
-template <bool BITS>
+template <bool BITS, bool KNOWN_BITS = false>
 __device__ __forceinline__ void mask_block_kv(float16_t& x, const FlexMask& m, const Mask2& visible, int qb, int kv,
                                               int Lq, int Lkv) {
-  if (!BITS || m.kind == FLEX_MASK_BAND) {
+  if (!KNOWN_BITS && (!BITS || m.kind == FLEX_MASK_BAND)) {
     const int dq = qb + m.q_offset - kv;                          // d = dq + off
     const int lo_off = clamp_big(m.lo) - dq;                      // off >= lo_off <=> d >= lo
     const int up = (kv < Lkv) ? (Lq - 1 - qb) : -1;               // off <= up <=> q < Lq (and the key exists)
