@@ -8,7 +8,7 @@
 // Two kernels.  fwd_mfma_kernel (any supported D, tile lists or not): one workgroup
 // (4 waves) per 128 query rows of one (batch, head), one 32-row block per wave; KV tiles of
 // 64 rows go through two LDS stages (register-prefetched one tile ahead, one workgroup
-// barrier per tile).  fwd_pipe_kernel (D = 64, no tile lists, nothing to mask): 256 query rows per
+// barrier per tile).  fwd_pipe_kernel (D = 64, no tile lists, a mask that hides nothing): 256 query rows per
 // workgroup, two blocks per wave, software-pipelined (see there).
 // Per 32-key step and 32-row block:
 //   S^T[kv, q]  = K_step . Q^T          D/16 v_mfma_f32_32x32x16
@@ -308,7 +308,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 // Tiles are fetched global -> LDS directly (no staging registers, no LDS stores),
 // one tile ahead of the one being read.
 // ---------------------------------------------------------------------------
-template <typename T, int KIND, bool ROUND_S>
+// TAIL: the key length is not a multiple of the tile; that instantiation masks the keys past the end in the last
+// tile.  The other one contains no mask code at all.
+template <typename T, int KIND, bool ROUND_S, bool TAIL>
 __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2) {
@@ -343,10 +345,10 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
     for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
   }
 
-  // every key tile is visited and nothing is masked: this kernel is launched for problems without tile
-  // lists, with a mask that hides nothing and a key length that is a multiple of the tile (mask code in
-  // the same function costs the unmasked path 3 %)
-  const int nt = p.Lkv / BN;
+  // every key tile is visited and nothing is masked but (TAIL) the keys past the end: this kernel is
+  // launched for problems without tile lists and with a mask that hides nothing (mask code in the same
+  // function costs the unmasked path 3 %, hence the two instantiations)
+  const int nt = TAIL ? (p.Lkv + BN - 1) / BN : p.Lkv / BN;
   auto tile_at = [&](int it) -> int { return it; };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
@@ -356,7 +358,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
   const int fill_row = lane >> 3;                         // row inside the 8-row group
   auto issue_tile = [&](int stage, int kv0) {
-    const int lim = p.Lkv - 1 - kv0;  // guard only: the key length is a multiple of the tile here
+    const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
     for (int j = 0; j < 2; j++) {
       const int r0 = 16 * w + 8 * j;
@@ -493,6 +495,21 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
           if (a == 1) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads (V columns)
           __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // six vector instructions
         }
+        if constexpr (TAIL) {
+          if (kv0 + BN > p.Lkv) {
+            // a real branch whose inputs pass through the asm, so that none of the mask
+            // arithmetic can be hoisted into the path of the complete tiles
+            int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+            asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+            const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
+                                             __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
+            if (cls == kBlockNone) fill_masked(s_cur);
+            else if (cls == kBlockMixed) {
+              const Mask2 visible(p.mask, b, h, p.Lkv);
+              mask_block_q<false>(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+            }
+          }
+        }
         // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
         float m_rel = xhalf_max(block_max(s_cur));
         const bool need = (m_rel > kTau) || (m_run[a] == -INFINITY && m_rel > -INFINITY);
@@ -578,12 +595,17 @@ static void launch_rs(const FlexAttnParams& p, const void* q, const void* k, con
   // longest one, which is what bounds a causal-like schedule.
   // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
   if constexpr (KIND != FLEX_SCORE_AFFINE) {
-    if (D == 64 && !p.tiles.kv_num && mask_hides_nothing(p.mask) && p.Lkv % kFwdBN == 0) {
+    if (D == 64 && !p.tiles.kv_num && mask_hides_nothing(p.mask)) {
       dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
-      if (p.flags & FLEX_ROUND_S)
-        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+      const bool tail = p.Lkv % kFwdBN != 0, rs = (p.flags & FLEX_ROUND_S) != 0;
+      if (rs && !tail)
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+      else if (rs)
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, true, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+      else if (!tail)
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
       else
-        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
+        hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, false, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v, (T*)o, lse2);
       return;
     }
   }
