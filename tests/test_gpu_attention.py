@@ -570,3 +570,37 @@ def test_softcap_saturates_cleanly(dev, D):
     assert rel_l2(out.detach().cpu(), want) <= 1e-3
     for got, w in ((qd.grad, wq), (kd.grad, wk), (vd.grad, wv)):
         assert rel_l2(got.cpu(), w) <= 2e-3 and max_abs(got.cpu(), w) <= 2e-2 * max(1.0, w.abs().max().item())
+
+
+def test_document_mask_equals_per_document_attention(dev):
+    """A document mask written as a plain callable over a captured tensor of document ids: the result must be what
+    ordinary attention gives on every document by itself (here torch's math-path SDPA in fp32 on the same device, an
+    implementation that shares nothing with the kernels or the oracle)."""
+    print("case document mask vs per-document attention", flush=True)
+    B, H, L, D = 2, 4, 1000, 64
+    lengths = [137, 400, 63, 400]
+    doc = torch.repeat_interleave(torch.arange(len(lengths)), torch.tensor(lengths)).to(dev)
+
+    def same_document(b, h, q_idx, kv_idx):
+        d = doc if q_idx.is_cuda else doc.cpu()
+        return d[q_idx.long()] == d[kv_idx.long()]
+    g = torch.Generator(device="cpu").manual_seed(9)
+    mk = lambda: torch.randn(B, H, L, D, generator=g, dtype=torch.float32).to(torch.float16).to(dev).requires_grad_(True)
+    q, k, v = mk(), mk(), mk()
+    d_o = torch.randn(B, H, L, D, generator=g, dtype=torch.float32).to(torch.float16).to(dev)
+    bm = fa.create_block_mask(same_document, 1, 1, L, L, device=dev)
+    out = fa.flax_attention(q, k, v, block_mask=bm)
+    out.backward(d_o)
+    qf, kf, vf = (t.detach().float().requires_grad_(True) for t in (q, k, v))
+    pieces, at = [], 0
+    from torch.nn.attention import SDPBackend, sdpa_kernel
+    with sdpa_kernel(SDPBackend.MATH):
+        for n in lengths:
+            s = slice(at, at + n)
+            pieces.append(torch.nn.functional.scaled_dot_product_attention(qf[:, :, s], kf[:, :, s], vf[:, :, s]))
+            at += n
+    want = torch.cat(pieces, dim=2)
+    want.backward(d_o.float())
+    assert rel_l2(out.detach().float().cpu(), want.detach().cpu()) <= 1e-3
+    for got, ref in ((q.grad, qf.grad), (k.grad, kf.grad), (v.grad, vf.grad)):
+        assert rel_l2(got.float().cpu(), ref.cpu()) <= 2e-3
