@@ -64,7 +64,7 @@ EXPORTS = [
     "flexattn_block_mask_workspace_bytes", "flexattn_block_mask_build",
     "flexattn_fwd_workspace_bytes", "flexattn_fwd",
     "flexattn_bwd_workspace_bytes", "flexattn_bwd",
-    "flexattn_decode_workspace_bytes", "flexattn_decode",
+    "flexattn_decode_workspace_bytes", "flexattn_decode", "flexattn_decode_static",
     "flexattn_probe_mfma",
     "flexattn_probe_mix",
     "flexattn_probe_read",
@@ -112,6 +112,7 @@ def lib() -> C.CDLL:
     L.flexattn_decode_workspace_bytes.restype = C.c_size_t
     L.flexattn_decode_workspace_bytes.argtypes = [C.POINTER(FlexAttnParams), C.c_int32]
     L.flexattn_decode.argtypes = [C.POINTER(FlexAttnParams)] + [C.c_void_p] * 5 + [C.c_int32, C.c_void_p, C.c_void_p]
+    L.flexattn_decode_static.argtypes = [C.POINTER(FlexAttnParams)] + [C.c_void_p] * 5 + [C.c_int32, C.c_void_p]
     L.flexattn_probe_mfma.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
     L.flexattn_probe_mix.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
     L.flexattn_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]

@@ -17,7 +17,14 @@
 //   the MFMA, so K and V are read once per group.
 // Each workgroup writes an unnormalised partial (O, m, l) per column; a second
 // kernel merges the splits:  O = sum_s 2^(m_s-m) O_s / sum_s 2^(m_s-m) l_s.
+#include <mutex>
 #include "mfma_common.cuh"
+
+// Split-KV partials of flexattn_decode_static: every GPU the library runs on holds its own copy of
+// this array, at its own address, until the process ends.  Host code never uses the array's name as
+// an address; flex_decode_static_scratch() asks the runtime for the device address once per device.
+constexpr size_t kStaticScratchBytes = FLEXATTN_DECODE_STATIC_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace flex {
 
@@ -423,6 +430,32 @@ int flex_decode_default_splits(const FlexAttnParams& p) {
 size_t flex_decode_workspace(const FlexAttnParams& p, int splits) {
   const size_t rows = (size_t)p.B * p.Hq * p.Lq;
   return (rows * splits * (p.D + 2) * sizeof(float) + 255) / 256 * 256;
+}
+
+// Device address of this file's scratch array on the current device, looked up once per device
+// (hipGetSymbolAddress neither allocates nor frees).  Returns nullptr with the error set on failure.
+void* flex_decode_static_scratch(size_t* bytes) {
+  constexpr int kMaxDev = 64;
+  static std::mutex mu;
+  static void* ptr_of[kMaxDev] = {};
+  *bytes = kStaticScratchBytes;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDev) {
+    flex_set_error("decode (static scratch): no usable current device (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr_of[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      flex_set_error("decode (static scratch): hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    ptr_of[dev] = ptr;
+  }
+  return ptr_of[dev];
 }
 
 int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,

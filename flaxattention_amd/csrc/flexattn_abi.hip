@@ -28,6 +28,7 @@ int flex_decode_default_splits(const FlexAttnParams& p);
 size_t flex_decode_workspace(const FlexAttnParams& p, int splits);
 int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
                        void* workspace, hipStream_t s);
+void* flex_decode_static_scratch(size_t* bytes);
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb);
 
 static int validate(const FlexAttnParams* p, const char* who) {
@@ -119,9 +120,38 @@ extern "C" size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32
   return flex_decode_workspace(*p, num_splits);
 }
 
+static int decode_checked(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
+                          int32_t num_splits, void* workspace, flexattn_stream_t stream);
+
 extern "C" int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                                int32_t num_splits, void* workspace, flexattn_stream_t stream) {
   if (int rc = validate(p, "flexattn_decode")) return rc;
+  return decode_checked(p, q, k, v, o, lse2, num_splits, workspace, stream);
+}
+
+extern "C" int flexattn_decode_static(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o,
+                                      float* lse2, int32_t num_splits, flexattn_stream_t stream) {
+  if (int rc = validate(p, "flexattn_decode_static")) return rc;
+  if (!flex_decode_supported(*p)) {
+    flex_set_error("flexattn_decode_static: needs fp16/bf16, D == Dv in {64,128}, Lq <= 64 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
+    return 1;
+  }
+  if (num_splits <= 0) num_splits = flex_decode_default_splits(*p);
+  const size_t need = flex_decode_workspace(*p, num_splits);
+  size_t cap = 0;
+  void* ws = flex_decode_static_scratch(&cap);
+  if (!ws) return 2;
+  if (need > cap) {
+    flex_set_error("flexattn_decode_static: %zu bytes of split-KV partials (B=%d Hq=%d Lq=%d D=%d, %d splits) exceed the "
+                   "built-in scratch of %zu bytes; use flexattn_decode with a caller workspace",
+                   need, p->B, p->Hq, p->Lq, p->D, num_splits, cap);
+    return 1;
+  }
+  return decode_checked(p, q, k, v, o, lse2, num_splits, ws, stream);
+}
+
+static int decode_checked(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
+                          int32_t num_splits, void* workspace, flexattn_stream_t stream) {
   if (p->q_index_base < 0 || p->q_index_base % 64 != 0) { flex_set_error("flexattn_decode: q_index_base must be a non-negative multiple of 64 (got %d)", p->q_index_base); return 1; }
   if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
   if (!flex_decode_supported(*p)) {

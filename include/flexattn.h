@@ -198,6 +198,20 @@ int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const
                     void* o, float* lse2, int32_t num_splits, void* workspace,
                     flexattn_stream_t stream);
 
+/* flexattn_decode for callers that cannot allocate device memory or hand in a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The split-KV partials go to a buffer of
+ * FLEXATTN_DECODE_STATIC_BYTES that is part of the library image on every GPU it runs on (held
+ * until the process ends); the call makes no hipMalloc / hipFree and no other allocating call.
+ * Problems whose partials (flexattn_decode_workspace_bytes) exceed that size are refused with
+ * an error; use flexattn_decode for those.  All calls on one GPU share the buffer, whose
+ * contents do not carry over between calls (every call overwrites what it reads): calls that
+ * overlap on one GPU -- two streams, two threads -- race.  Results are bit-identical to
+ * flexattn_decode with the same num_splits.  */
+#define FLEXATTN_DECODE_STATIC_BYTES ((size_t)16 << 20)
+int flexattn_decode_static(const FlexAttnParams* p, const void* q, const void* k, const void* v,
+                           void* o, float* lse2, int32_t num_splits, flexattn_stream_t stream);
+
 /* Measurement aid with no counterpart in the reference: launches a kernel that only
  * issues v_mfma_f32_32x32x16_f16 on pseudo-random operands (512 workgroups x 4 waves,
  * 8*iters MFMAs per wave) so that a caller can time the matrix throughput the GPU
