@@ -244,49 +244,66 @@ def pmc_probe(dev, name, opts):
     torch.cuda.synchronize()
 
 
+_probe_lib = None
+
+
+def probe_lib():
+    """libflexprobe.so: bench-only measurement kernels (MFMA-only, instruction-mix and streaming-read), built next to
+    the product library by the same Makefile but no part of it."""
+    global _probe_lib
+    if _probe_lib is None:
+        from flaxattention_amd import _lib
+        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libflexprobe.so")
+        L = C.CDLL(path)
+        L.flexprobe_last_error.restype = C.c_char_p
+        L.flexprobe_mfma.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
+        L.flexprobe_mix.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
+        L.flexprobe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]
+        _probe_lib = L
+    return _probe_lib
+
+
+def probe_check(rc, who):
+    if rc:
+        raise RuntimeError(f"{who} failed ({rc}): {probe_lib().flexprobe_last_error().decode()}")
+
+
 def run_mfma_probe(dev):
-    """Matrix throughput this GPU sustains on a kernel that only issues fp16 MFMAs on pseudo-random operands
-    (the library's measurement aid): the practical ceiling next to the published peak."""
-    from flaxattention_amd import _lib
-    L = _lib.lib()
+    """Matrix throughput this GPU sustains on a kernel that only issues fp16 MFMAs on pseudo-random operands:
+    the practical ceiling next to the published peak."""
+    L = probe_lib()
     sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
     flops = C.c_double(0.0)
     stream = torch.cuda.current_stream(dev).cuda_stream
 
     def go():
-        rc = L.flexattn_probe_mfma(sink.data_ptr(), 4096, C.byref(flops), stream)
-        if rc:
-            _lib.check(rc, "flexattn_probe_mfma")
+        probe_check(L.flexprobe_mfma(sink.data_ptr(), 4096, C.byref(flops), stream), "flexprobe_mfma")
     us = event_time_us(go, 20)
     return flops.value / us / 1e6
 
 
 def run_mix_probe(dev):
-    """Matrix flop rate of the library's instruction-mix probe: 8, 12 or 16 MFMAs interleaved with the vector work of
+    """Matrix flop rate of the instruction-mix probe: 8, 12 or 16 MFMAs interleaved with the vector work of
     one 32x32 score block (80 FMAs + 16 exponentials), two waves per SIMD.  The ceiling of a fused attention step of
     that mix on this GPU: 8 = forward at D 64, 12 = dQ kernel, 16 = dK/dV kernel and forward at D 128."""
-    from flaxattention_amd import _lib
-    L = _lib.lib()
+    L = probe_lib()
     sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
     flops = C.c_double(0.0)
     stream = torch.cuda.current_stream(dev).cuda_stream
     out = {}
     for nm in (8, 12, 16):
         def go():
-            rc = L.flexattn_probe_mix(sink.data_ptr(), 2048, nm, C.byref(flops), stream)
-            if rc:
-                _lib.check(rc, "flexattn_probe_mix")
+            probe_check(L.flexprobe_mix(sink.data_ptr(), 2048, nm, C.byref(flops), stream), "flexprobe_mix")
         us = event_time_us(go, 20)
         out[str(nm)] = round(flops.value / us / 1e6, 1)
     return out
 
 
 def run_read_probe(dev):
-    """Read rate of the library's bare streaming-read kernel over 268 MB (the K + V bytes of one decode call of
+    """Read rate of the bare streaming-read kernel over 268 MB (the K + V bytes of one decode call of
     configuration 5): rotating over three buffers, which no launch finds in the 256 MB last-level cache, and
     re-reading one buffer.  GB/s."""
-    from flaxattention_amd import _lib
-    L = _lib.lib()
+    L = probe_lib()
     nbytes = 2 * 8 * 8 * 16384 * 64 * 2
     bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(3)]
     sink = torch.zeros(65536, dtype=torch.float32, device=dev)
@@ -294,10 +311,9 @@ def run_read_probe(dev):
     turn = [0]
 
     def go(n_bufs):
-        rc = L.flexattn_probe_read(bufs[turn[0] % n_bufs].data_ptr(), nbytes, sink.data_ptr(), stream)
+        rc = L.flexprobe_read(bufs[turn[0] % n_bufs].data_ptr(), nbytes, sink.data_ptr(), 0, 0, stream)
         turn[0] += 1
-        if rc:
-            _lib.check(rc, "flexattn_probe_read")
+        probe_check(rc, "flexprobe_read")
     cold = event_time_us(lambda: go(3), 30)
     warm = event_time_us(lambda: go(1), 30)
     return {"rotating_buffers": round(nbytes / cold / 1e3), "one_buffer": round(nbytes / warm / 1e3)}

@@ -17,7 +17,7 @@ CSRC_DIR = os.path.join(_HERE, "csrc")
 FLEX_F32, FLEX_F16, FLEX_BF16 = 0, 1, 2
 SCORE_IDENTITY, SCORE_CHECKERBOARD, SCORE_ALIBI, SCORE_TANH_SOFTCAP, SCORE_REL_BIAS, SCORE_AFFINE = range(6)
 MASK_BAND, MASK_BITS = 0, 1
-FLAG_ROUND_S, FLAG_STRICT, FLAG_FORCE_GENERIC, FLAG_BWD_ONLY_DQ, FLAG_BWD_ONLY_DKV = 1, 2, 4, 8, 16
+FLAG_ROUND_S, FLAG_STRICT, FLAG_FORCE_GENERIC, FLAG_BWD_ONLY_DQ, FLAG_BWD_ONLY_DKV, FLAG_PARITY = 1, 2, 4, 8, 16, 32
 INT_MIN, INT_MAX = -(2 ** 31), 2 ** 31 - 1
 
 
@@ -56,7 +56,8 @@ class FlexAttnParams(C.Structure):
                 ("v_stride", C.c_int64 * 3), ("o_stride", C.c_int64 * 3),
                 ("scale", C.c_float), ("flags", C.c_int32),
                 ("score", FlexScoreMod), ("mask", FlexMask), ("tiles", FlexTileLists),
-                ("tiles_bwd", FlexTileLists), ("q_index_base", C.c_int32), ("pad_", C.c_int32)]
+                ("tiles_bwd", FlexTileLists), ("q_index_base", C.c_int32), ("pad_", C.c_int32),
+                ("d_lse2", C.c_void_p)]
 
 
 EXPORTS = [
@@ -65,9 +66,6 @@ EXPORTS = [
     "flexattn_fwd_workspace_bytes", "flexattn_fwd",
     "flexattn_bwd_workspace_bytes", "flexattn_bwd",
     "flexattn_decode_workspace_bytes", "flexattn_decode", "flexattn_decode_static",
-    "flexattn_probe_mfma",
-    "flexattn_probe_mix",
-    "flexattn_probe_read",
 ]
 
 _lib: Optional[C.CDLL] = None
@@ -113,9 +111,6 @@ def lib() -> C.CDLL:
     L.flexattn_decode_workspace_bytes.argtypes = [C.POINTER(FlexAttnParams), C.c_int32]
     L.flexattn_decode.argtypes = [C.POINTER(FlexAttnParams)] + [C.c_void_p] * 5 + [C.c_int32, C.c_void_p, C.c_void_p]
     L.flexattn_decode_static.argtypes = [C.POINTER(FlexAttnParams)] + [C.c_void_p] * 5 + [C.c_int32, C.c_void_p]
-    L.flexattn_probe_mfma.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
-    L.flexattn_probe_mix.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
-    L.flexattn_probe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     _lib = L
     return L
 

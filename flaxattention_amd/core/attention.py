@@ -10,9 +10,19 @@ forward saves (q, k, v, out, lse2), backward returns (dq, dk, dv).
 
 ``kernel_options`` (accepted and ignored by the reference, attention.py:179)
 selects numerics here:
-    {"strict": True}    faithful kernels: S, normalised P, dP and dS are
-                        rounded through the input dtype exactly where the
-                        reference's dense path rounds them
+    {"numerics": "parity" | "fast"}   fused (matrix-core) kernels, 16-bit inputs:
+                        "parity": the rounding points of the reference's dense
+                        path -- S rounded to the input dtype (attention.py:27),
+                        the NORMALISED P rounded before P.V (attention.py:104-105;
+                        a two-pass forward), and in the backward dP rounded,
+                        delta = sum_j P round(dP), dS rounded after scaling.
+                        "fast": one-pass online softmax (the unnormalised P is
+                        rounded), delta = sum_d O dO, dP kept in fp32; about 1.5x
+                        faster.  Default: "parity" for bfloat16, whose 8-bit
+                        mantissa puts "fast" 3e-3 (relative L2) away from the dense
+                        path, and "fast" for float16, where it stays within 1e-3.
+    {"strict": True}    faithful kernels on the vector ALU: the same rounding
+                        points as "parity", any dtype and head size
     {"round_s": bool}   fused kernels: round Q.K^T through the input dtype
                         (default True, as attention.py:27 computes that product
                         in the input dtype)
@@ -149,6 +159,11 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
         flags |= _lib.FLAG_ROUND_S
     if opts.get("backend", "auto") == "generic":
         flags |= _lib.FLAG_FORCE_GENERIC
+    numerics = opts.get("numerics", "parity" if q.dtype == torch.bfloat16 else "fast")
+    if numerics not in ("parity", "fast"):
+        raise ValueError(f'kernel_options["numerics"] must be "parity" or "fast", got {numerics!r}')
+    if numerics == "parity" and q.dtype != torch.float32:
+        flags |= _lib.FLAG_PARITY
     plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, score, flags, opts))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and opts.get("tile_lists", True) and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
@@ -248,13 +263,16 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     return o, lse2
 
 
-def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o) -> Tuple[Array, Array, Array]:
+def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o, d_lse2=None) -> Tuple[Array, Array, Array]:
     L = _lib.lib()
     d_o = d_o.contiguous()
+    if d_lse2 is not None:
+        d_lse2 = d_lse2.to(torch.float32).contiguous()
     dq = torch.empty((plan.B, plan.Hq, plan.Lq, plan.D), dtype=q.dtype, device=q.device)
     dk = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.D), dtype=q.dtype, device=q.device)
     dv = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.Dv), dtype=q.dtype, device=q.device)
     p = plan.params(q, k, v, o)
+    p.d_lse2 = d_lse2.data_ptr() if d_lse2 is not None else None
     with torch.cuda.device(q.device):
         ws = torch.empty(max(L.flexattn_bwd_workspace_bytes(p), 256), dtype=torch.uint8, device=q.device)
         rc = L.flexattn_bwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), d_o.data_ptr(),
@@ -269,13 +287,17 @@ class _FlexAttention(torch.autograd.Function):
         o, lse2 = _run_fwd(plan, q, k, v)
         ctx.save_for_backward(q, k, v, o, lse2)
         ctx.plan = plan
-        ctx.mark_non_differentiable(lse2)
+        ctx.set_materialize_grads(False)   # an output the loss does not use arrives as None, not as zeros
         return o, lse2
 
     @staticmethod
-    def backward(ctx, d_o, _d_lse):
+    def backward(ctx, d_o, d_lse2):
+        # the log-sum-exp is a differentiable output as in the reference (attention.py:97-106): its cotangent
+        # joins the softmax's row term inside the kernels
         q, k, v, o, lse2 = ctx.saved_tensors
-        dq, dk, dv = _run_bwd(ctx.plan, q, k, v, o, lse2, d_o)
+        if d_o is None:
+            d_o = torch.zeros_like(o)
+        dq, dk, dv = _run_bwd(ctx.plan, q, k, v, o, lse2, d_o, d_lse2)
         return dq, dk, dv, None
 
 

@@ -248,16 +248,20 @@ class BlockMask:
             if Qp >= Lq and W * 32 >= Lkv and Bm in (1, B) and Hm in (1, H):
                 return s
         self.spec = resolve_mask_mod(self.mask_mod, B, H, Lq, Lkv, device)
+        self._tile_cache.clear()   # lists made from the previous lowering describe another batch / head extent
         return self.spec
 
     def tile_lists(self, q_block: int, kv_block: int, B: int, H: int, Lq: int, Lkv: int, device):
         """Ordered tile lists at the kernels' own granularity (built once per
         granularity from the mask functor and cached)."""
+        spec = self.resolved_spec(B, H, Lq, Lkv, device)
         key = (q_block, kv_block, (Lq + q_block - 1) // q_block, (Lkv + kv_block - 1) // kv_block)
         hit = self._tile_cache.get(key)
-        if hit is not None:
+        # lists are indexed by (batch, head) with stride 0 for an extent of 1: cached ones serve this call only if
+        # their extents are 1 or the call's own (a mask built for B=2 used with a batch of 4 is rebuilt from its
+        # functor, as the reference would simply evaluate the mask_mod for all four)
+        if hit is not None and hit["spec"] is spec and hit["B"] in (1, B) and hit["H"] in (1, H):
             return hit
-        spec = self.resolved_spec(B, H, Lq, Lkv, device)
         Bm, Hm = (1, 1)
         if spec.bits is not None:
             Bm, Hm = spec.bits.shape[0], spec.bits.shape[1]

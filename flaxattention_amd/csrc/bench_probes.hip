@@ -1,3 +1,10 @@
+// Bench-only measurement kernels (no counterpart in the reference and no part of the product
+// library): built into libflexprobe.so, which only bench.py and a GPU test load.
+//   flexprobe_mfma   nothing but v_mfma_f32_32x32x16_f16 on pseudo-random operands
+//   flexprobe_mix    the instruction mix of a fused attention step
+//   flexprobe_read   a bare streaming read
+// Each returns 0 on success; flexprobe_last_error() gives the message otherwise.
+//
 // Measurement aid (no counterpart in the reference): a kernel that does nothing but
 // v_mfma_f32_32x32x16_f16 on pseudo-random operands, two waves per SIMD, four independent
 // accumulators per wave.  Timing it gives the matrix throughput this GPU sustains under its
@@ -91,51 +98,76 @@ __global__ __launch_bounds__(256, 2) void mix_probe_kernel(float* __restrict__ s
 
 }  // namespace flex
 
-void flex_set_error(const char* fmt, ...);
+#include <cstdarg>
+#include <cstdio>
+static thread_local char g_probe_err[256] = "";
+static void flex_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_probe_err, sizeof(g_probe_err), fmt, ap);
+  va_end(ap);
+}
+extern "C" const char* flexprobe_last_error(void) { return g_probe_err; }
 
 namespace flex {
-// A streaming read and nothing else: every thread folds 16-byte loads (four independent ones per trip) into a value
-// that is practically never written.
+// A streaming read and nothing else: every thread folds NLD independent 16-byte loads per trip into a value that
+// is practically never written.  Consecutive threads read consecutive 16-byte pieces; a workgroup walks the buffer
+// in strides of the whole grid, so at any time the grid covers one contiguous window.
+template <int NLD>
 __global__ __launch_bounds__(256) void read_probe_kernel(const uint4* __restrict__ src, size_t n_vec, float* __restrict__ sink) {
   const size_t tid = blockIdx.x * (size_t)blockDim.x + threadIdx.x, total = (size_t)gridDim.x * blockDim.x;
   uint4 acc = make_uint4(0, 0, 0, 0);
-  for (size_t i = tid; i < n_vec; i += 4 * total) {
-    const uint4 z = make_uint4(0, 0, 0, 0);
-    const uint4 a = src[i], b = i + total < n_vec ? src[i + total] : z;
-    const uint4 c = i + 2 * total < n_vec ? src[i + 2 * total] : z, d = i + 3 * total < n_vec ? src[i + 3 * total] : z;
-    acc.x ^= a.x ^ b.x ^ c.x ^ d.x; acc.y ^= a.y ^ b.y ^ c.y ^ d.y;
-    acc.z ^= a.z ^ b.z ^ c.z ^ d.z; acc.w ^= a.w ^ b.w ^ c.w ^ d.w;
+  for (size_t i = tid; i < n_vec; i += NLD * total) {
+    uint4 x[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; j++) x[j] = i + j * total < n_vec ? src[i + j * total] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NLD; j++) { acc.x ^= x[j].x; acc.y ^= x[j].y; acc.z ^= x[j].z; acc.w ^= x[j].w; }
   }
   if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x12345678u) sink[tid & 0xffff] = 1.f;
 }
 }  // namespace flex
 
-// 1024 workgroups of 256 threads (the grid a bare read is fastest with here) over `bytes` of device memory.
-extern "C" int flexattn_probe_read(const void* src, size_t bytes, float* sink, void* stream) {
+// `workgroups` x 256 threads over `bytes` of device memory, `loads_in_flight` (1, 2, 4, 8 or 16) independent 16-byte
+// loads per thread and trip.  workgroups <= 0: 1024; loads_in_flight <= 0: 4.  `sink`: 65536 floats.
+extern "C" int flexprobe_read(const void* src, size_t bytes, float* sink, int32_t workgroups, int32_t loads_in_flight, void* stream) {
   if (!src || !sink || bytes < 16 || ((uintptr_t)src & 15)) {
-    flex_set_error("flexattn_probe_read: needs a 16-byte aligned device buffer of at least 16 bytes and a sink of 65536 floats");
+    flex_set_error("flexprobe_read: needs a 16-byte aligned device buffer of at least 16 bytes and a sink of 65536 floats");
     return 1;
   }
-  hipLaunchKernelGGL(flex::read_probe_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, (const uint4*)src, bytes / 16, sink);
+  if (workgroups <= 0) workgroups = 1024;
+  if (loads_in_flight <= 0) loads_in_flight = 4;
+  const dim3 grid(workgroups), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const uint4* s4 = (const uint4*)src;
+  const size_t n = bytes / 16;
+  switch (loads_in_flight) {
+    case 1: hipLaunchKernelGGL(flex::read_probe_kernel<1>, grid, block, 0, st, s4, n, sink); break;
+    case 2: hipLaunchKernelGGL(flex::read_probe_kernel<2>, grid, block, 0, st, s4, n, sink); break;
+    case 4: hipLaunchKernelGGL(flex::read_probe_kernel<4>, grid, block, 0, st, s4, n, sink); break;
+    case 8: hipLaunchKernelGGL(flex::read_probe_kernel<8>, grid, block, 0, st, s4, n, sink); break;
+    case 16: hipLaunchKernelGGL(flex::read_probe_kernel<16>, grid, block, 0, st, s4, n, sink); break;
+    default: flex_set_error("flexprobe_read: loads_in_flight must be 1, 2, 4, 8 or 16"); return 1;
+  }
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { flex_set_error("flexattn_probe_read: launch failed: %s", hipGetErrorString(e)); return 2; }
+  if (e != hipSuccess) { flex_set_error("flexprobe_read: launch failed: %s", hipGetErrorString(e)); return 2; }
   return 0;
 }
 
 // 512 workgroups of 4 waves (two waves per SIMD on 256 compute units), 8 * iters MFMAs per wave.
-extern "C" int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, void* stream) {
-  if (!sink || iters <= 0) { flex_set_error("flexattn_probe_mfma: needs a device buffer of 512*256 floats and iters > 0"); return 1; }
+extern "C" int flexprobe_mfma(float* sink, int32_t iters, double* flops_per_launch, void* stream) {
+  if (!sink || iters <= 0) { flex_set_error("flexprobe_mfma: needs a device buffer of 512*256 floats and iters > 0"); return 1; }
   hipLaunchKernelGGL(flex::mfma_probe_kernel, dim3(512), dim3(256), 0, (hipStream_t)stream, sink, iters);
   if (flops_per_launch) *flops_per_launch = 512.0 * 4 * 8.0 * iters * 2.0 * 32 * 32 * 16;
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { flex_set_error("flexattn_probe_mfma: launch failed: %s", hipGetErrorString(e)); return 2; }
+  if (e != hipSuccess) { flex_set_error("flexprobe_mfma: launch failed: %s", hipGetErrorString(e)); return 2; }
   return 0;
 }
 
 // Same grid; `iters` units of `mfma_per_unit` (8, 12 or 16) matrix instructions + 96 vector instructions per wave.
-extern "C" int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch, void* stream) {
+extern "C" int flexprobe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch, void* stream) {
   if (!sink || iters <= 0 || (mfma_per_unit != 8 && mfma_per_unit != 12 && mfma_per_unit != 16)) {
-    flex_set_error("flexattn_probe_mix: needs a device buffer of 512*256 floats, iters > 0 and mfma_per_unit in {8, 12, 16}");
+    flex_set_error("flexprobe_mix: needs a device buffer of 512*256 floats, iters > 0 and mfma_per_unit in {8, 12, 16}");
     return 1;
   }
   hipStream_t st = (hipStream_t)stream;
@@ -144,6 +176,6 @@ extern "C" int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_u
   else hipLaunchKernelGGL(flex::mix_probe_kernel<16>, dim3(512), dim3(256), 0, st, sink, iters, 0.999f, 0.001f);
   if (flops_per_launch) *flops_per_launch = 512.0 * 4 * (double)mfma_per_unit * iters * 2.0 * 32 * 32 * 16;
   hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { flex_set_error("flexattn_probe_mix: launch failed: %s", hipGetErrorString(e)); return 2; }
+  if (e != hipSuccess) { flex_set_error("flexprobe_mix: launch failed: %s", hipGetErrorString(e)); return 2; }
   return 0;
 }

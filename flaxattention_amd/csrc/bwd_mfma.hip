@@ -1,680 +1,14 @@
-// Fused flash-attention backward for gfx950 (fp16 / bf16, D = Dv in {64, 128}).
-//
-// Takes the place of _preprocess_backward + mha_backward_kernel
-// (flaxattention/kernel/attention.py:338-553) and of jax.grad through the dense
-// path.  P is recomputed from the saved base-2 log-sum-exp.  Two kernels:
-//
-//  bwd_dq_kernel   one workgroup per 128 query rows, sweeping KV tiles of 128 (64 at D = 128;
-//                  the entries of the 128-granular backward lists), fetched global -> LDS
-//                  directly into two stages.  Transposed products keep one query
-//                  row per lane, so lse and delta are per-lane scalars:
-//                    S^T = K.Q^T,  dP^T = V.dO^T,  dS^T = P^T o (dP^T - delta) * g,
-//                    dQ^T += K^T.dS^T.
-//                  Also produces delta_i = sum_d O_id dO_id for the second kernel.
-//  bwd_dkv_kernel  one workgroup per 128 key rows, sweeping query tiles of 128
-//                  from the transposed tile lists.  Here a lane owns one key
-//                  row: S = Q.K^T, dP = dO.V^T, dV^T += dO^T.P, dK^T += Q^T.dS.
-//                  Four waves = four key blocks of 32 rows.  With GQA the
-//                  workgroup loops over the query heads of its group.
-#include "mfma_common.cuh"
-
-namespace flex {
-
-constexpr int kBM = 128;     // query tile (list granularity)
-constexpr int kBN = 128;     // key tile staged per step by the dQ kernel at D = 64 (half of it at D = 128)
-constexpr int kListBN = 128; // key granularity of the backward tile lists = key rows of a dK/dV workgroup
-
-// MASKED = false: the caller guarantees that there is nothing to mask (no tile lists, a mask that hides nothing,
-// key length a multiple of the tile); that instantiation carries no mask code, which is worth 2 % on its own.
-template <typename T, int D, int KIND, bool ROUND_S, bool MASKED>
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
-                                                      const T* __restrict__ k, const T* __restrict__ v,
-                                                      const T* __restrict__ o, const float* __restrict__ lse2,
-                                                      const T* __restrict__ d_o, T* __restrict__ dq,
-                                                      float* __restrict__ delta_out) {
-  typedef typename Frag<T>::vec8 vec8;
-  // keys staged per step: 128 at D = 64, 64 at D = 128, so that two stages of K and V are 64 KB
-  // either way and two workgroups (two waves per SIMD) share a compute unit
-  constexpr int BM = kBM, BN = D == 64 ? kBN : kBN / 2;
-  constexpr int DS = D / 16, DB = D / 32, CPR = D / 8;
-  constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
-  constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor
-  // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled
-  // rows): while one tile is consumed the next one lands, one workgroup barrier per tile
-  __shared__ __align__(16) T Ksm[2][BN * D];
-  __shared__ __align__(16) T Vsm[2][BN * D];
-
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
-  const int nqt = (p.Lq + BM - 1) / BM;
-  int rank, bh;
-  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
-  const int qt = nqt - 1 - rank;
-  const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
-  const int q_row = qt * BM + w * 32 + i32;
-  const int q_ld = min(q_row, p.Lq - 1);
-  const int64_t row_id = ((int64_t)b * p.Hq + h) * p.Lq + q_ld;
-
-  vec8 qf[DS], dof[DS];
-  float dpart = 0.f;
-  {
-    const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
-    const T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_ld * p.o_stride[2] + 8 * g;
-    const T* dop = d_o + row_id * D + 8 * g;  // dO is contiguous [B,Hq,Lq,D]
-#pragma unroll
-    for (int s = 0; s < DS; s++) {
-      qf[s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
-      dof[s] = *reinterpret_cast<const vec8*>(dop + 16 * s);
-      vec8 of = *reinterpret_cast<const vec8*>(op + 16 * s);
-#pragma unroll
-      for (int e = 0; e < 8; e++) dpart = fmaf((float)of[e], (float)dof[s][e], dpart);
-    }
-  }
-  const float delta = xhalf_sum(dpart);
-  if (q_row < p.Lq && g == 0) delta_out[row_id] = delta;
-  float lse = lse2[row_id];
-  if (lse == -INFINITY) lse = INFINITY;  // row without visible keys: P = 0
-
-  const FlexTileLists& tl = p.tiles_bwd;
-  const int32_t* full_idx = nullptr;
-  const int32_t* part_idx = nullptr;
-  int n_full, n_part = 0;
-  if (tl.kv_num) {
-    const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
-    n_full = tl.full_kv_num[row];
-    n_part = tl.kv_num[row];
-    full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
-    part_idx = tl.kv_idx + row * tl.n_kv_blocks;
-  } else {
-    // no lists: every tile is visited, and evaluated under a mask that can hide something
-    n_full = (p.Lkv + BN - 1) / BN;
-    if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
-  }
-  // a list entry covers `sub` staged tiles of BN keys (the lists are kListBN-granular);
-  // the schedule below runs over (entry, part) pairs flattened into one index
-  const int sub = full_idx ? tl.kv_block / BN : 1;
-  const int nt = (n_full + n_part) * sub;
-  const int n_full_t = n_full * sub;
-  auto tile_at = [&](int it) -> int {
-    if (!full_idx) return it;
-    const int e = sub == 2 ? (it >> 1) : it, part = sub == 2 ? (it & 1) : 0;
-    return (e < n_full ? full_idx[e] : part_idx[e - n_full]) * sub + part;
-  };
-
-  const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
-  const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
-  const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
-  // tile fetch: wave w fills rows [32w, 32w + 32) of the K and the V tile, RPI rows per instruction;
-  // the lane that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
-  const int fill_row = lane / CPR, fill_pos = lane % CPR;
-  auto issue_tile = [&](int stage, int kv0) {
-    const int lim = p.Lkv - 1 - kv0;  // rows past the end: clamped (finite filler, masked out below)
-#pragma unroll
-    for (int j = 0; j < NI; j++) {
-      const int r0 = (BN / 4) * w + RPI * j;
-      const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);  // the wave's first row is a multiple of 16
-      const int row = min(r0 + fill_row, lim);
-      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
-      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
-                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
-    }
-  };
-  // element offsets inside a 32-row block: row fragments (row i32, chunk 2s + g sits at (2s) ^ kz) and
-  // transposing reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
-  const int kz = g ^ lds_swz<D>(i32);
-  int toff[2][DB];
-  {
-    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
-#pragma unroll
-    for (int e = 0; e < 2; e++)
-#pragma unroll
-      for (int db = 0; db < DB; db++) {
-        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
-        toff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
-      }
-  }
-
-  Score2<KIND> sm;
-  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
-  Mask2 visible(p.mask, b, h, p.Lkv);
-  float16_t dqacc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; db++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) dqacc[db][r] = 0.f;
-
-  int t_cur = nt > 0 ? tile_at(0) : 0;
-  int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) issue_tile(0, t_cur * BN);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __syncthreads();
-  const float neg_delta = -delta;
-  for (int it = 0; it < nt; it++) {
-    const int kv0 = t_cur * BN;
-    const bool masked = MASKED && ((it >= n_full_t) || (kv0 + BN > p.Lkv));
-    const T* Ks = Ksm[it & 1];
-    const T* Vs = Vsm[it & 1];
-    if (it + 1 < nt) {
-      // the other stage was last read before the previous barrier: the next tile lands there
-      // while this one is consumed; the tile index after that is looked up a tile ahead
-      issue_tile((it + 1) & 1, t_nxt * BN);
-      t_cur = t_nxt;
-      if (it + 2 < nt) t_nxt = tile_at(it + 2);
-    }
-
-    // one 32-key block at a time (S, dP, softmax, dQ): half the accumulator registers of
-    // doing both blocks side by side
-#pragma unroll
-    for (int nb = 0; nb < BN / 32; nb++) {
-      // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
-      // entirely hidden (nothing to do)
-      int cls = kBlockAll;
-      if (masked) {
-        cls = block_class(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
-        if (cls == kBlockNone) continue;
-      }
-      sm.tile(q_row, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
-      // dP starts at -delta, so the accumulator comes out as dP - delta
-      float16_t sacc, dpacc, gacc;
-#pragma unroll
-      for (int r = 0; r < 16; r++) { sacc[r] = 0.f; dpacc[r] = neg_delta; }
-      const T* kp = Ks + (nb * 32 + i32) * D;
-      const T* vp = Vs + (nb * 32 + i32) * D;
-#pragma unroll
-      for (int s = 0; s < DS; s++) {
-        sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(kp + (((2 * s) ^ kz) * 8)), qf[s], sacc);
-        dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(vp + (((2 * s) ^ kz) * 8)), dof[s], dpacc);
-      }
-      // x = log2(e) * score_mod(scale * s) - lse  (P = 2^x); g = d score_mod / d score kept for later
-#pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float s0 = sacc[r], s1 = sacc[r + 1];
-        if (ROUND_S) round_pair<T>(s0, s1);
-        sacc[r] = sm.apply_sub(s0, acc_row(r), lse);
-        sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), lse);
-        if (!Score2<KIND>::kGradOne) {
-          gacc[r] = sm.grad(s0, acc_row(r));
-          gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
-        }
-      }
-      if (cls == kBlockMixed) {
-        // a real branch whose inputs pass through the asm, so that none of the mask
-        // arithmetic can be hoisted into the unmasked path
-        int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
-        asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
-        mask_block_q(sacc, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
-      }
-      vec8 dsf[2];
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        typename Pair<T>::v2 pr[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int r = 8 * tt + 2 * e;
-          float d0 = fast_exp2(sacc[r]) * dpacc[r];
-          float d1 = fast_exp2(sacc[r + 1]) * dpacc[r + 1];
-          if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
-          pr[e] = Pair<T>::pack(d0, d1);
-        }
-        dsf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
-      }
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          const T* ktp = Ks + (32 * nb + 16 * tt) * D;
-          short4_t lo = lds_read_tr(ktp + toff[0][db]);
-          short4_t hi = lds_read_tr(ktp + toff[1][db]);
-          dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[tt], dqacc[db]);
-        }
-      }
-    }
-    // this wave's share of the next tile has landed; after the barrier everyone's has
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-  }
-
-  // the scale factor of dS = P o (dP - delta) o g * scale is applied once here
-  if (q_row < p.Lq) {
-    T* op = dq + row_id * D + 4 * g;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int rr = 0; rr < 4; rr++) {
-        union { T e[4]; uint2 u; } pk;
-#pragma unroll
-        for (int e = 0; e < 4; e++) pk.e[e] = (T)(dqacc[db][4 * rr + e] * p.scale);
-        *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
-      }
-  }
-}
-
-extern __shared__ __align__(16) unsigned char bwd_smem[];
-
-// dK/dV workgroup: 4 waves = 4 key blocks of 32 rows (kListBN keys); every wave takes the
-// four 32-row query blocks of a tile in turn, so a Q / dO tile fetched from L2 serves 128 keys
-// and nothing has to be summed across waves.  With D = 64 two such workgroups share a
-// compute unit (two waves per SIMD); being independent they drift out of phase, so one's
-// matrix work overlaps the other's vector work and barrier waits.
-template <int D> struct DkvShape {
-  static constexpr int kWaves = kListBN / 32;
-  static constexpr int kThreads = kWaves * 64;
-  static constexpr int kQBlocks = kBM / 32;        // 32-row query blocks per wave and tile
-  static constexpr int kStages = D == 64 ? 2 : 1;  // LDS stages of the query-side tiles
-};
-
-// BITS: the mask is a bitmap.  Band masks get an instantiation of their own, without the bitmap code: with it in the
-// same function the compiler allocates registers differently and the unmasked path runs 5 % slower.
-template <typename T, int D, int KIND, bool ROUND_S, bool BITS>
-__global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
-                                                               const T* __restrict__ k, const T* __restrict__ v,
-                                                               const float* __restrict__ lse2,
-                                                               const float* __restrict__ delta,
-                                                               const T* __restrict__ d_o, T* __restrict__ dk,
-                                                               T* __restrict__ dv) {
-  typedef typename Frag<T>::vec8 vec8;
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  constexpr int BM = kBM, BN = kListBN;
-  constexpr int kDkvThreads = DkvShape<D>::kThreads, QBW = DkvShape<D>::kQBlocks;
-  // D = 64: the Q and dO tiles land in LDS straight from global memory (unpadded rows, chunk c of row r at
-  // position c ^ lds_swz(r): conflict-free for the row-fragment and the transposing reads); D = 128 stages them
-  // through registers into padded rows
-  constexpr bool DIRECT = D == 64;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = DIRECT ? D : D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
-  // LDS stages of (Q tile, dO tile, lse, -delta).  D = 64 keeps two, so that one workgroup
-  // barrier per tile suffices; with D = 128 a second stage would cost the second workgroup
-  // of the compute unit, so one stage is refilled between two barriers.
-  constexpr int NSTG = DkvShape<D>::kStages;
-  constexpr int kStageBytes = 2 * BM * ROWE * (int)sizeof(T) + 2 * BM * (int)sizeof(float);
-  auto stage_q = [&](int st) { return reinterpret_cast<T*>(bwd_smem + st * kStageBytes); };
-
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
-  const int wk = __builtin_amdgcn_readfirstlane(w);  // key block (32 rows) of this wave (wave-uniform)
-  const int nkt = (p.Lkv + BN - 1) / BN;
-  int kt, bh;  // early key tiles see the most queries under causal masks
-  xcd_tile_map(blockIdx.x, nkt, p.Hkv * p.B, kt, bh);
-  const int hk = bh % p.Hkv, b = bh / p.Hkv, G = p.Hq / p.Hkv;
-  const int kv_col = kt * BN + wk * 32 + i32;
-  const int kv_ld = min(kv_col, p.Lkv - 1);
-
-  vec8 kf[DS], vf[DS];
-  {
-    const T* kp = k + b * p.k_stride[0] + hk * p.k_stride[1] + (int64_t)kv_ld * p.k_stride[2] + 8 * g;
-    const T* vp = v + b * p.v_stride[0] + hk * p.v_stride[1] + (int64_t)kv_ld * p.v_stride[2] + 8 * g;
-#pragma unroll
-    for (int s = 0; s < DS; s++) {
-      kf[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
-      vf[s] = *reinterpret_cast<const vec8*>(vp + 16 * s);
-    }
-  }
-  float16_t dkacc[DB], dvacc[DB];
-#pragma unroll
-  for (int db = 0; db < DB; db++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
-  // element offsets inside a 32-row block of a tile: row fragments (row i32, chunk 2s + g) and transposing
-  // reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
-  const int kz = DIRECT ? (g ^ lds_swz<D>(i32)) : g;
-  int toff[2][DB];
-  {
-    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
-#pragma unroll
-    for (int e = 0; e < 2; e++)
-#pragma unroll
-      for (int db = 0; db < DB; db++) {
-        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
-        const int pos = DIRECT ? (chunk ^ lds_swz<D>(rl + 8 * e)) : chunk;
-        toff[e][db] = (rl + 8 * e) * ROWE + pos * 8 + 4 * (i16 & 1);
-      }
-  }
-
-  const FlexTileLists& tl = p.tiles_bwd;
-  Score2<KIND> sm;
-  float key_grad = 1.f;  // derivative of a score_mod that depends on the key only: applied to dK at the end
-
-  for (int gi = 0; gi < G; gi++) {
-    const int h = hk * G + gi;
-    sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
-    const int32_t* full_idx = nullptr;
-    const int32_t* part_idx = nullptr;
-    int n_full, n_part = 0;
-    if (tl.kv_num) {
-      const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_kv_blocks + kt;
-      n_full = tl.full_q_num[row];
-      n_part = tl.q_num[row];
-      full_idx = tl.full_q_idx + row * tl.n_q_blocks;
-      part_idx = tl.q_idx + row * tl.n_q_blocks;
-    } else {
-      // no lists: every tile is visited, and evaluated under a mask that can hide something
-      n_full = (p.Lq + BM - 1) / BM;
-      if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
-    }
-    const int nt = n_full + n_part;
-    const T* qbase = q + b * p.q_stride[0] + h * p.q_stride[1];
-    const int64_t rows0 = ((int64_t)b * p.Hq + h) * p.Lq;
-    const T* dobase = d_o + rows0 * D;
-
-    auto tile_at = [&](int it) -> int {
-      if (!full_idx) return it;
-      return it < n_full ? full_idx[it] : part_idx[it - n_full];
-    };
-    u32x4 qreg[DIRECT ? 1 : NLD], oreg[DIRECT ? 1 : NLD];
-    float lreg = INFINITY, dreg = 0.f;
-    // direct fetch: wave w fills rows [32w, 32w + 32) of the Q and the dO tile, 8 rows per instruction; the lane
-    // that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
-    auto issue_tile = [&](int st, int q0) {
-      T* Qw = stage_q(st);
-      T* Ow = Qw + BM * ROWE;
-      const int lim = p.Lq - 1 - q0;  // rows past the end: clamped (finite filler; their lse is +inf, so P = 0)
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int r0 = 32 * w + 8 * j;
-        const int chunk = (lane & 7) ^ lds_swz<D>(8 * j + (lane >> 3));  // the wave's first row is a multiple of 16
-        const int row = min(r0 + (lane >> 3), lim);
-        const T* qg = qbase + (int64_t)(q0 + row) * p.q_stride[2] + chunk * 8;
-        const T* og = dobase + (int64_t)(q0 + row) * D + chunk * 8;
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)qg,
-                                         (__attribute__((address_space(3))) void*)(Qw + r0 * ROWE), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)og,
-                                         (__attribute__((address_space(3))) void*)(Ow + r0 * ROWE), 16, 0, 0);
-      }
-    };
-    auto load_tile = [&](int q0) {
-      if constexpr (!DIRECT) {
-#pragma unroll
-        for (int j = 0; j < NLD; j++) {
-          const int c = tid + kDkvThreads * j, r = min(c / CPR, p.Lq - 1 - q0), cc = c % CPR;  // clamped: finite filler
-          qreg[j] = *reinterpret_cast<const u32x4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
-          oreg[j] = *reinterpret_cast<const u32x4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
-        }
-      }
-      lreg = INFINITY;
-      dreg = 0.f;
-      if (tid < BM && q0 + tid < p.Lq) {
-        lreg = lse2[rows0 + q0 + tid];
-        dreg = delta[rows0 + q0 + tid];
-        if (lreg == -INFINITY) lreg = INFINITY;  // row without visible keys: P = 0
-      }
-    };
-    int t_cur = nt > 0 ? tile_at(0) : 0;
-    int t_nxt = nt > 1 ? tile_at(1) : 0;
-    auto store_tile = [&](int st) {
-      T* Qw = stage_q(st);
-      T* Ow = Qw + BM * ROWE;
-      float* lw = reinterpret_cast<float*>(Ow + BM * ROWE);
-      if constexpr (!DIRECT) {
-#pragma unroll
-        for (int j = 0; j < NLD; j++) {
-          const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
-          *reinterpret_cast<u32x4*>(Qw + r * ROWE + cc * 8) = qreg[j];
-          *reinterpret_cast<u32x4*>(Ow + r * ROWE + cc * 8) = oreg[j];
-        }
-      }
-      if (tid < BM) {
-        lw[tid] = lreg;        // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
-        lw[BM + tid] = -dreg;  // the dP accumulator starts from -delta
-      }
-    };
-    __syncthreads();  // the stages may still be in use by the previous head of the group
-    if (nt > 0) {
-      if constexpr (DIRECT) issue_tile(0, t_cur * BM);
-      load_tile(t_cur * BM);
-    }
-    if (NSTG == 2) {
-      if (nt > 0) store_tile(0);
-      if (nt > 1) load_tile(t_nxt * BM);
-      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-    }
-    for (int it = 0; it < nt; it++) {
-      const int q0 = t_cur * BM;
-      const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
-      const int st = NSTG == 2 ? (it & 1) : 0;
-      const T* Qs = stage_q(st);
-      const T* Os = Qs + BM * ROWE;
-      const float* lse_s = reinterpret_cast<const float*>(Os + BM * ROWE);
-      const float* del_s = lse_s + BM;
-      if (NSTG == 2) {
-        if (it + 1 < nt) {
-          // the other stage was last read before the previous barrier: refill it (D = 64: the
-          // tile itself is fetched straight into it now and awaited at the end of this tile; lse
-          // and delta, like whole tiles at D = 128, were prefetched into registers), then start
-          // fetching the one after
-          if constexpr (DIRECT) issue_tile((it + 1) & 1, t_nxt * BM);
-          store_tile((it + 1) & 1);
-          t_cur = t_nxt;
-          if (it + 2 < nt) {
-            t_nxt = tile_at(it + 2);
-            load_tile(t_nxt * BM);
-          }
-        }
-      } else {
-        store_tile(0);  // the barrier that closed the previous tile freed the stage
-        __syncthreads();
-        if (it + 1 < nt) load_tile(t_nxt * BM);
-        t_cur = t_nxt;
-        if (it + 2 < nt) t_nxt = tile_at(it + 2);
-      }
-
-#pragma unroll
-      for (int qs = 0; qs < QBW; qs++) {
-      // ---- S = Q.K^T and dP = dO.V^T for 32 query rows x 32 keys ----
-      const int qrow_w = qs * 32;
-      int cls = kBlockAll;
-      if (masked) {
-        if constexpr (BITS) {
-          const Mask2 visible(p.mask, b, h, p.Lkv);
-          cls = block_class(p.mask, visible, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
-        } else {
-          cls = band_block_class(p.mask, q0 + qrow_w, kt * BN + wk * 32, p.Lq, p.Lkv);
-        }
-        if (cls == kBlockNone) continue;
-      }
-      float16_t sacc, dpacc;
-      const int ql = qrow_w + 4 * g;  // local row of register 0
-      sm.tileT(q0 + ql, kv_col);      // a table-reading score_mod fetches its entries under the products
-#pragma unroll
-      for (int rr = 0; rr < 4; rr++) {
-        const float4_t d4 = *reinterpret_cast<const float4_t*>(del_s + ql + 8 * rr);
-#pragma unroll
-        for (int e = 0; e < 4; e++) { sacc[4 * rr + e] = 0.f; dpacc[4 * rr + e] = d4[e]; }
-      }
-      {
-        const T* qp = Qs + (qrow_w + i32) * ROWE;
-        const T* op = Os + (qrow_w + i32) * ROWE;
-#pragma unroll
-        for (int s = 0; s < DS; s++) {
-          sacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(qp + (((2 * s) ^ kz) * 8)), kf[s], sacc);
-          dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + (((2 * s) ^ kz) * 8)), vf[s], dpacc);
-        }
-      }
-      // D = 64 has the registers to fetch the transposed dO and Q fragments of the closing products now, under the
-      // softmax arithmetic, instead of right before their use (1.7 % of the kernel's time)
-      vec8 a_do[2][DB], a_q[2][DB];
-      if constexpr (DIRECT) {
-#pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-          for (int db = 0; db < DB; db++) {
-            const int base = (qrow_w + 16 * tt) * ROWE;
-            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
-            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
-          }
-      }
-      // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
-      float16_t gacc;
-      if constexpr (KIND == kScoreCheckerboardKv) key_grad = sm.key_grad;
-#pragma unroll
-      for (int rr = 0; rr < 4; rr++) {
-        const float4_t l4 = *reinterpret_cast<const float4_t*>(lse_s + ql + 8 * rr);
-#pragma unroll
-        for (int e = 0; e < 4; e += 2) {
-          const int r = 4 * rr + e;
-          float s0 = sacc[r], s1 = sacc[r + 1];
-          if (ROUND_S) round_pair<T>(s0, s1);
-          sacc[r] = sm.apply_sub(s0, acc_row(r), l4[e]);
-          sacc[r + 1] = sm.apply_sub(s1, acc_row(r + 1), l4[e + 1]);
-          if (!Score2<KIND>::kGradOne) {
-            gacc[r] = sm.grad(s0, acc_row(r));
-            gacc[r + 1] = sm.grad(s1, acc_row(r + 1));
-          }
-        }
-      }
-      if (cls == kBlockMixed) {
-        int q_opaque = q0 + ql, kv_opaque = kv_col;
-        asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));  // keeps the mask arithmetic behind this branch
-        const Mask2 visible(p.mask, b, h, p.Lkv);
-        mask_block_kv<BITS>(sacc, p.mask, visible, q_opaque, kv_opaque, p.Lq, p.Lkv);
-      }
-      vec8 pf[2], dsf[2];
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-        typename Pair<T>::v2 pp[4], dd[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int r = 8 * tt + 2 * e;
-          const float p0 = fast_exp2(sacc[r]), p1 = fast_exp2(sacc[r + 1]);
-          float d0 = p0 * dpacc[r], d1 = p1 * dpacc[r + 1];
-          if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
-          pp[e] = Pair<T>::pack(p0, p1);
-          dd[e] = Pair<T>::pack(d0, d1);
-        }
-        pf[tt] = join_pairs<T>(pp[0], pp[1], pp[2], pp[3]);
-        dsf[tt] = join_pairs<T>(dd[0], dd[1], dd[2], dd[3]);
-      }
-      // ---- dV^T += dO^T.P, dK^T += Q^T.dS (contraction over this wave's 32 query rows) ----
-#pragma unroll
-      for (int tt = 0; tt < 2; tt++) {
-#pragma unroll
-        for (int db = 0; db < DB; db++) {
-          const int base = (qrow_w + 16 * tt) * ROWE;
-          if constexpr (!DIRECT) {
-            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
-            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
-          }
-          dvacc[db] = Frag<T>::mfma(a_do[tt][db], pf[tt], dvacc[db]);
-          dkacc[db] = Frag<T>::mfma(a_q[tt][db], dsf[tt], dkacc[db]);
-        }
-      }
-      }  // query blocks of this wave
-      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed
-      __syncthreads();
-    }
-  }
-
-  if (kv_col < p.Lkv) {
-    const int64_t row_id = ((int64_t)b * p.Hkv + hk) * p.Lkv + kv_col;
-    T* dkp = dk + row_id * D + 4 * g;
-    T* dvp = dv + row_id * D + 4 * g;
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-      for (int rr = 0; rr < 4; rr++) {
-        union { T e[4]; uint2 u; } pk, pv;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          const int r = 4 * rr + e;
-          pk.e[e] = (T)(dkacc[db][r] * (p.scale * key_grad));  // the scale factor of dS is applied once here
-          pv.e[e] = (T)dvacc[db][r];
-        }
-        *reinterpret_cast<uint2*>(dkp + 32 * db + 8 * rr) = pk.u;
-        *reinterpret_cast<uint2*>(dvp + 32 * db + 8 * rr) = pv.u;
-      }
-  }
-}
-
-template <int D, typename T> constexpr size_t dkv_smem() {
-  return DkvShape<D>::kStages * ((size_t)2 * kBM * (D == 64 ? D : D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
-}
-
-template <typename T, int D, int KIND, bool RS, bool BITS>
-static int launch_dkv_as(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
-                         void* dk, void* dv, float* delta, hipStream_t s) {
-  constexpr size_t sm = dkv_smem<D, T>();
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS, BITS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm);
-    if (e != hipSuccess) return 2;
-    attr_set = true;
-  }
-  const int nkt = (p.Lkv + kListBN - 1) / kListBN;
-  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS, BITS>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, s, p,
-                     (const T*)q, (const T*)k, (const T*)v, lse2, delta, (const T*)d_o, (T*)dk, (T*)dv);
-  return 0;
-}
-template <typename T, int D, int KIND, bool RS>
-static int launch_dkv(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
-                      void* dk, void* dv, float* delta, hipStream_t s) {
-  if (p.mask.kind == FLEX_MASK_BITS) return launch_dkv_as<T, D, KIND, RS, true>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
-  return launch_dkv_as<T, D, KIND, RS, false>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
-}
-
-template <typename T, int D, int KIND, bool RS>
-static void launch_dq(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                      const void* d_o, void* dq, float* delta, hipStream_t s) {
-  const int nqt = (p.Lq + kBM - 1) / kBM;
-  constexpr int BN = D == 64 ? kBN : kBN / 2;   // the kernel's key tile
-  const dim3 grid(nqt * p.Hq * p.B);
-  if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0)
-    hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS, false>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v,
-                       (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
-  else
-    hipLaunchKernelGGL((bwd_dq_kernel<T, D, KIND, RS, true>), grid, dim3(256), 0, s, p, (const T*)q, (const T*)k, (const T*)v,
-                       (const T*)o, lse2, (const T*)d_o, (T*)dq, delta);
-}
-
-template <typename T, int D, int KIND, bool RS>
-static int launch_one(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                      const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  if (!(p.flags & FLEX_BWD_ONLY_DKV)) {
-    if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.p0 > 0.f && p.score.p1 > 0.f) {
-      // positive factors: the derivative folds into the exponent
-      constexpr int KF = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardFold : KIND;
-      launch_dq<T, D, KF, RS>(p, q, k, v, o, lse2, d_o, dq, delta, s);
-    } else {
-      launch_dq<T, D, KIND, RS>(p, q, k, v, o, lse2, d_o, dq, delta, s);
-    }
-  }
-  if (p.flags & FLEX_BWD_ONLY_DQ) return 0;
-  if (KIND == FLEX_SCORE_CHECKERBOARD && p.score.i0) {
-    // keyed on the key index: the derivative is constant along a lane's dK row
-    constexpr int KV = KIND == FLEX_SCORE_CHECKERBOARD ? kScoreCheckerboardKv : KIND;
-    return launch_dkv<T, D, KV, RS>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
-  }
-  return launch_dkv<T, D, KIND, RS>(p, q, k, v, lse2, d_o, dk, dv, delta, s);
-}
-
-template <typename T, int D, int KIND>
-static int launch_rs(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                     const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  if (p.flags & FLEX_ROUND_S) return launch_one<T, D, KIND, true>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-  return launch_one<T, D, KIND, false>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-}
-
-template <typename T, int D>
-static int launch_kind(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                       const void* d_o, void* dq, void* dk, void* dv, float* delta, hipStream_t s) {
-  switch (p.score.kind) {
-    case FLEX_SCORE_IDENTITY: return launch_rs<T, D, FLEX_SCORE_IDENTITY>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-    case FLEX_SCORE_CHECKERBOARD: return launch_rs<T, D, FLEX_SCORE_CHECKERBOARD>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-    case FLEX_SCORE_ALIBI: return launch_rs<T, D, FLEX_SCORE_ALIBI>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-    case FLEX_SCORE_TANH_SOFTCAP: return launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-    case FLEX_SCORE_REL_BIAS: return launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-    case FLEX_SCORE_AFFINE: return launch_rs<T, D, FLEX_SCORE_AFFINE>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-  }
-  return 1;
-}
-
-}  // namespace flex
+// Fused flash-attention backward for gfx950 (fp16 / bf16, D = Dv in {64, 128}): checks and dispatch.  The kernels are
+// in bwd_mfma.cuh, instantiated per (dtype, head size) by bwd_mfma_inst.hip.
+#include "bwd_mfma.cuh"
 
 using namespace flex;
 void flex_set_error(const char* fmt, ...);
 bool flex_mfma_shape_ok(const FlexAttnParams& p);
+int flex_mfma_bwd_f16_64(const FlexAttnParams& p, const BwdArgs& a);
+int flex_mfma_bwd_f16_128(const FlexAttnParams& p, const BwdArgs& a);
+int flex_mfma_bwd_bf16_64(const FlexAttnParams& p, const BwdArgs& a);
+int flex_mfma_bwd_bf16_128(const FlexAttnParams& p, const BwdArgs& a);
 
 bool flex_mfma_bwd_supported(const FlexAttnParams& p) {
   if (!flex_mfma_shape_ok(p)) return false;
@@ -693,12 +27,10 @@ int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const v
     flex_set_error("fused backward needs 16-byte aligned tensors");
     return 1;
   }
-  float* delta = (float*)workspace;
+  const BwdArgs a = {q, k, v, o, d_o, lse2, dq, dk, dv, (float*)workspace, s};
   int rc;
-  if (p.dtype == FLEX_F16) rc = p.D == 64 ? launch_kind<f16, 64>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s)
-                                          : launch_kind<f16, 128>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
-  else rc = p.D == 64 ? launch_kind<bf16, 64>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s)
-                      : launch_kind<bf16, 128>(p, q, k, v, o, lse2, d_o, dq, dk, dv, delta, s);
+  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_mfma_bwd_f16_64(p, a) : flex_mfma_bwd_f16_128(p, a);
+  else rc = p.D == 64 ? flex_mfma_bwd_bf16_64(p, a) : flex_mfma_bwd_bf16_128(p, a);
   if (rc == 1) flex_set_error("fused backward: unsupported score_mod kind %d", p.score.kind);
   if (rc == 2) flex_set_error("fused backward: could not raise the dynamic LDS limit");
   return rc;

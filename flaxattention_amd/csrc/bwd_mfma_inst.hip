@@ -1,0 +1,6 @@
+// One (dtype, head size) instantiation of the fused backward kernels.  The Makefile compiles this file once per
+// combination (FLEX_T = f16 | bf16, FLEX_D = 64 | 128, FLEX_FN = the exported launcher's name), so that the four sets
+// of kernels build in parallel.
+#include "bwd_mfma.cuh"
+
+int FLEX_FN(const FlexAttnParams& p, const flex::BwdArgs& a) { return flex::launch_kind<flex::FLEX_T, FLEX_D>(p, a); }

@@ -65,7 +65,7 @@ static int check_launch(const char* who) {
   return 0;
 }
 
-extern "C" int flexattn_abi_version(void) { return 2; }
+extern "C" int flexattn_abi_version(void) { return 3; }
 extern "C" const char* flexattn_last_error(void) { return g_err; }
 
 extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t which, int32_t* qb, int32_t* kvb) {
@@ -76,7 +76,24 @@ extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, in
   return 0;
 }
 
-extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) { return 0; }
+// FLEX_PARITY asks for the reference's rounding points.  The fused kernels have a mode for it; where only the
+// generic kernels apply, FLEX_STRICT is the same numerics.
+static FlexAttnParams with_parity_resolved(const FlexAttnParams* p, bool fused) {
+  FlexAttnParams r = *p;
+  if (r.flags & FLEX_PARITY) {
+    if (fused) r.flags |= FLEX_ROUND_S;
+    else r.flags = (r.flags & ~FLEX_PARITY) | FLEX_STRICT;
+  }
+  return r;
+}
+static bool wants_fused(const FlexAttnParams* p) { return !(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)); }
+
+static size_t lse_bytes(const FlexAttnParams* p) { return ((size_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256; }
+
+extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
+  // the two passes of the parity numerics hand the log-sum-exp over in lse2, or here when the caller wants no lse2
+  return (p && (p->flags & FLEX_PARITY)) ? lse_bytes(p) : 0;
+}
 
 extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                             void* workspace, flexattn_stream_t stream) {
@@ -85,8 +102,17 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o) { flex_set_error("flexattn_fwd: null tensor pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
-  if (!(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)) && flex_mfma_fwd_supported(*p)) rc = flex_mfma_fwd(*p, q, k, v, o, lse2, s);
-  else rc = flex_generic_fwd(*p, q, k, v, o, lse2, s);
+  const bool fused = wants_fused(p) && flex_mfma_fwd_supported(*p);
+  const FlexAttnParams pr = with_parity_resolved(p, fused);
+  if (fused) {
+    if ((pr.flags & FLEX_PARITY) && !lse2) {
+      if (!workspace) { flex_set_error("flexattn_fwd: FLEX_PARITY needs lse2 or a workspace of flexattn_fwd_workspace_bytes()"); return 1; }
+      lse2 = (float*)workspace;
+    }
+    rc = flex_mfma_fwd(pr, q, k, v, o, lse2, s);
+  } else {
+    rc = flex_generic_fwd(pr, q, k, v, o, lse2, s);
+  }
   if (rc) return rc;
   return check_launch("flexattn_fwd");
 }
@@ -108,8 +134,10 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o || !lse2 || !d_o || !dq || !dk || !dv || !workspace) { flex_set_error("flexattn_bwd: null pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
-  if (!(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)) && flex_mfma_bwd_supported(*p)) rc = flex_mfma_bwd(*p, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s);
-  else rc = flex_generic_bwd(*p, q, k, v, lse2, d_o, dq, dk, dv, (float*)workspace, s);
+  const bool fused = wants_fused(p) && flex_mfma_bwd_supported(*p);
+  const FlexAttnParams pr = with_parity_resolved(p, fused);
+  if (fused) rc = flex_mfma_bwd(pr, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s);
+  else rc = flex_generic_bwd(pr, q, k, v, lse2, d_o, dq, dk, dv, (float*)workspace, s);
   if (rc) return rc;
   return check_launch("flexattn_bwd");
 }

@@ -1,0 +1,695 @@
+// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128}).
+//
+// Takes the place of mha_forward_kernel (flaxattention/kernel/attention.py:
+// 34-149) and of the dense math path (flaxattention/core/attention.py:14-106)
+// for 16-bit inputs, with a real online softmax and with skipping of masked-out
+// KV tiles, which the reference computes but never uses.
+//
+// Two kernels.  fwd_mfma_kernel (any supported D, tile lists or not): one workgroup
+// (4 waves) per 128 query rows of one (batch, head), one 32-row block per wave; KV tiles of
+// 64 rows go through two LDS stages (register-prefetched one tile ahead, one workgroup
+// barrier per tile).  fwd_pipe_kernel (D = 64, no tile lists, a mask that hides nothing): 256 query rows per
+// workgroup, two blocks per wave, software-pipelined (see there).
+// Per 32-key step and 32-row block:
+//   S^T[kv, q]  = K_step . Q^T          D/16 v_mfma_f32_32x32x16
+//   online softmax in the accumulator layout: a lane holds 16 of the 32 scores
+//   of ONE query row, the other 16 sit in lane ^ 32 -> row max/sum are
+//   in-register reductions plus one permlane32 swap; the reference maximum only
+//   moves when it is beaten by 2^8, so the accumulator is rarely rescaled
+//   O^T[d, q] += V_step^T . P^T         D/16 v_mfma (P^T is already in B-operand
+//   layout; V^T fragments come from transposing LDS reads)
+#pragma once
+#include "mfma_common.cuh"
+
+namespace flex {
+
+constexpr int kFwdBN = 64;
+constexpr int kFwdBM = 128;   // query rows of a list-driven workgroup = q granularity of the forward lists
+constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dense kernel (D = 64, no lists)
+
+// BITS: the mask is a bitmap.  Band masks get an instantiation of their own, without the bitmap code and the scalar
+// registers its pointers and strides occupy.
+//
+// PASS selects the numerics:
+//   kFwdOnePass  online softmax; the unnormalised P is rounded to the input dtype for the P.V product
+//   kFwdLse      first pass of the parity numerics: only the base-2 log-sum-exp of every row (no V, no P.V)
+//   kFwdNorm     second pass: P = 2^(x - lse2) is the normalised probability, rounded to the input dtype and
+//                multiplied into V as it is -- what the dense path computes (attention.py:104-105 normalises in
+//                fp32, casts P to the input dtype and then multiplies)
+enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2 };
+template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
+__global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                           const T* __restrict__ k, const T* __restrict__ v,
+                                                           T* __restrict__ o, float* __restrict__ lse2) {
+  typedef typename Frag<T>::vec8 vec8;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int RQ = 1, BM = kFwdBM, BN = kFwdBN;
+  constexpr int DS = D / 16;     // k-steps of the Q.K^T product
+  constexpr int DB = D / 32;     // 32-row blocks of O^T
+  constexpr int ROWE = D + 8;    // LDS row length in elements (16 B of padding)
+  constexpr int CPR = D / 8;     // 16-byte chunks per row
+  constexpr int NLD = BN * CPR / 256;  // chunks per thread per tile
+  // two LDS stages: while one tile is consumed the next one is written, so a
+  // single workgroup barrier per tile suffices
+  __shared__ __align__(16) T Ksm[2][BN * ROWE];
+  __shared__ __align__(16) T Vsm[PASS == kFwdLse ? 1 : 2][PASS == kFwdLse ? 8 : BN * ROWE];
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
+  const int nqt = (p.Lq + BM - 1) / BM;
+  int rank, bh;
+  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
+  const int qt = nqt - 1 - rank;  // late query tiles see the most keys under causal masks
+  const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
+
+  // this lane's query rows: block a sits at q_row0 + 32 * a
+  const int q_row0 = qt * BM + w * (32 * RQ) + i32;
+
+  // Q fragments (B operand of S^T = K.Q^T), resident for the whole kernel
+  vec8 qf[RQ][DS];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_ld = min(q_row0 + 32 * a, p.Lq - 1);
+    const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+  }
+
+  // tile schedule
+  const FlexTileLists& tl = p.tiles;
+  const int32_t* full_idx = nullptr;
+  const int32_t* part_idx = nullptr;
+  int n_full, n_part = 0;
+  if (tl.kv_num) {
+    const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
+    n_full = tl.full_kv_num[row];
+    n_part = tl.kv_num[row];
+    full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
+    part_idx = tl.kv_idx + row * tl.n_kv_blocks;
+  } else {
+    // no lists: every tile is visited, and evaluated under a mask that can hide something
+    n_full = (p.Lkv + BN - 1) / BN;
+    if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
+  }
+  const int nt = n_full + n_part;
+  auto tile_at = [&](int it) -> int {
+    if (!full_idx) return it;
+    return it < n_full ? full_idx[it] : part_idx[it - n_full];
+  };
+
+  const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
+  const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
+  const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
+
+  u32x4 kreg[NLD], vreg[NLD];
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
+      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
+      if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+    }
+  };
+  auto store_tile = [&](int stage) {
+#pragma unroll
+    for (int j = 0; j < NLD; j++) {
+      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
+      if constexpr (PASS != kFwdLse) *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
+    }
+  };
+
+  Score2<KIND> sm;
+  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
+
+  float16_t oacc[RQ][DB];
+  float m_run[RQ], l_run[RQ];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    m_run[a] = -INFINITY;
+    l_run[a] = 0.f;
+    if constexpr (PASS == kFwdNorm) {
+      // the row's log-sum-exp from the first pass takes the place of the running reference maximum and never
+      // moves; a row without visible keys (-inf) gets +inf, so that every P is 0
+      const float l2 = lse2[((int64_t)b * p.Hq + h) * p.Lq + min(q_row0 + 32 * a, p.Lq - 1)];
+      m_run[a] = l2 == -INFINITY ? INFINITY : l2;
+    }
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[a][db][r] = 0.f;
+  }
+
+  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  int t_cur = nt > 0 ? tile_at(0) : 0;
+  int t_nxt = nt > 1 ? tile_at(1) : 0;
+  // prologue: tile 0 into stage 0, tile 1 into registers
+  if (nt > 0) {
+    load_tile(t_cur * BN);
+    store_tile(0);
+  }
+  if (nt > 1) load_tile(t_nxt * BN);
+  __syncthreads();
+  for (int it = 0; it < nt; it++) {
+    const int kv0 = t_cur * BN;
+    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
+    const T* Ks = Ksm[it & 1];
+    const T* Vs = Vsm[PASS == kFwdLse ? 0 : (it & 1)];
+    t_cur = t_nxt;
+    if (it + 2 < nt) t_nxt = tile_at(it + 2);
+
+    // Each 32-row half of the tile is one online-softmax step.
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+      // most 32x32 blocks of a partial tile are entirely visible (no mask evaluation) or
+      // entirely hidden (the step is skipped)
+      int cls = kBlockAll;
+      if (masked) {
+        if constexpr (BITS) {
+          const Mask2 visible(p.mask, b, h, p.Lkv);
+          cls = block_class<true>(p.mask, visible, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        } else {
+          cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_row0 - i32), kv0 + nb * 32, 0x7fffffff, p.Lkv);
+        }
+      }
+      if (cls != kBlockNone) {
+      sm.tile(q_row0, kv0 + nb * 32 + 4 * g);  // a table-reading score_mod fetches its entries under the products
+      // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
+      vec8 kfr[DS], vfr[2][DB];
+      {
+        const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+#pragma unroll
+        for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+        if constexpr (PASS != kFwdLse) {
+#pragma unroll
+          for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+              const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
+              vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+            }
+        }
+      }
+      // ---- S^T = K . Q^T for every query block of the wave ----
+      float16_t sacc[RQ];
+#pragma unroll
+      for (int a = 0; a < RQ; a++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) sacc[a][r] = 0.f;
+#pragma unroll
+      for (int s = 0; s < DS; s++)
+#pragma unroll
+        for (int a = 0; a < RQ; a++) sacc[a] = Frag<T>::mfma(kfr[s], qf[a][s], sacc[a]);
+
+      // The query blocks of the wave go through each phase together: their
+      // dependency chains (max tree, lane-half swap, exp) are independent and
+      // interleave, and one branch covers the rare rescale of either block.
+      float m_use[RQ], m_rel[RQ];
+      bool need[RQ], any_need = false;
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        const int q_row = q_row0 + 32 * a;
+        // ---- score_mod relative to the running reference max, tile mask where needed ----
+        m_use[a] = (PASS != kFwdNorm && m_run[a] == -INFINITY) ? 0.f : m_run[a];
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float s0 = sacc[a][r], s1 = sacc[a][r + 1];
+          if (ROUND_S) round_pair<T>(s0, s1);
+          sacc[a][r] = sm.apply_sub(s0, acc_row(r), m_use[a]);
+          sacc[a][r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use[a]);
+        }
+        if (cls == kBlockMixed) {
+          // a real branch: every input of the mask arithmetic passes through this asm, so that
+          // none of it can be hoisted into the unmasked path (it costs as much as the softmax)
+          int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+          asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+          const Mask2 visible(p.mask, b, h, p.Lkv);
+          mask_block_q<BITS, BITS>(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+        }
+      }
+      // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
+      if constexpr (PASS != kFwdNorm) {
+#pragma unroll
+      for (int a = 0; a < RQ; a++) m_rel[a] = block_max(sacc[a]);
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        m_rel[a] = xhalf_max(m_rel[a]);
+        need[a] = (m_rel[a] > kTau) || (m_run[a] == -INFINITY && m_rel[a] > -INFINITY);
+        any_need |= need[a];
+      }
+      }
+      if (PASS != kFwdNorm && __any(any_need)) {
+#pragma unroll
+        for (int a = 0; a < RQ; a++) {
+          float m_opaque = m_rel[a];
+          asm volatile("" : "+v"(m_opaque));  // keeps this rare path a real branch (never if-converted)
+          const float delta = need[a] ? m_opaque : 0.f;
+          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
+          m_run[a] = need[a] ? (m_use[a] + m_rel[a]) : m_run[a];
+          l_run[a] *= alpha;
+#pragma unroll
+          for (int r = 0; r < 16; r++) sacc[a][r] -= delta;
+          if constexpr (PASS == kFwdOnePass) {
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+              for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
+          }
+        }
+      }
+      if constexpr (PASS == kFwdLse) {
+        // only the row sums, in fp32 (the dense path sums the unrounded exponentials)
+#pragma unroll
+        for (int a = 0; a < RQ; a++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) l_run[a] += fast_exp2(sacc[a][r]);
+      } else {
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        vec8 pf[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+          typename Pair<T>::v2 pr[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p0 = fast_exp2(sacc[a][8 * tt + 2 * e]);
+            const float p1 = fast_exp2(sacc[a][8 * tt + 2 * e + 1]);
+            pr[e] = Pair<T>::pack(p0, p1);
+            if constexpr (PASS == kFwdOnePass) l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+          }
+          pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        }
+        // ---- O^T += V^T . P^T (issued before the next block's exponentials so the two overlap) ----
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+      }
+      }  // not the log-sum-exp pass
+      }  // block not entirely hidden
+      if (nb == 0 && it + 1 < nt) {
+        // the other stage was last read before the previous barrier: refill it with the
+        // tile prefetched into registers, then start fetching the one after
+        store_tile((it + 1) & 1);
+        if (it + 2 < nt) load_tile(t_nxt * BN);
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue ----
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_row = q_row0 + 32 * a;
+    const float l_tot = PASS == kFwdNorm ? 1.f : xhalf_sum(l_run[a]);
+    const float inv = PASS == kFwdNorm ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);  // kFwdNorm: P came normalised
+    if (q_row < p.Lq) {
+      if constexpr (PASS != kFwdLse) {
+        T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_row * p.o_stride[2] + 4 * g;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int rr = 0; rr < 4; rr++) {
+            union { T e[4]; uint2 u; } pk;
+#pragma unroll
+            for (int e = 0; e < 4; e++) pk.e[e] = (T)(oacc[a][db][4 * rr + e] * inv);
+            *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
+          }
+      }
+      if (PASS != kFwdNorm && lse2 && g == 0)
+        lse2[((int64_t)b * p.Hq + h) * p.Lq + q_row] = l_tot > 0.f ? m_run[a] + log2f(l_tot) : -INFINITY;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// D = 64: software-pipelined variant.  A wave owns two blocks of 32 query rows
+// and walks "units" (32-key step, query block).  The instruction stream of a
+// unit pairs every group of matrix instructions with independent vector work,
+// so that the matrix pipe and the vector ALU of a SIMD run at the same time
+// even when the waves of a workgroup march in lockstep:
+//   region A: scale / score_mod of S(u)            ||  S^T = K.Q^T of unit u+1
+//   (tile mask if needed, row max, rare rescale of the accumulator)
+//   region B: exponentials, rounding, row sum      ||  O^T += V^T.P^T of unit u-1
+// Every matrix result is first read at least half a unit after it was issued.
+// Unit u-1 and unit u+1 belong to the wave's other query block, so a rescale in
+// unit u never touches an accumulator that a matrix instruction is writing.
+// KV tiles go through three LDS stages with one workgroup barrier per tile: a
+// stage is refilled only after a barrier that follows its last fragment read.
+// Tiles are fetched global -> LDS directly (no staging registers, no LDS stores),
+// one tile ahead of the one being read.
+// ---------------------------------------------------------------------------
+// TAIL: the key length is not a multiple of the tile; that instantiation masks the keys past the end in the last
+// tile.  The other one contains no mask code at all.
+template <typename T, int KIND, bool ROUND_S, bool TAIL>
+__global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, const T* __restrict__ q,
+                                                           const T* __restrict__ k, const T* __restrict__ v,
+                                                           T* __restrict__ o, float* __restrict__ lse2) {
+  typedef typename Frag<T>::vec8 vec8;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  constexpr int D = 64, RQ = 2, BM = kPipeBM, BN = kFwdBN;
+  constexpr int DS = D / 16, DB = D / 32;
+  // KV tiles land in LDS straight from global memory (global_load_lds, 16 bytes per lane, a wave
+  // instruction fills 8 rows of 128 bytes), so rows are unpadded; the 16-byte chunk c of row r is
+  // kept at chunk position c ^ lds_swz(r), which makes both the row-fragment reads and the
+  // transposing reads conflict-free.  The lane that fills position (r, pos) therefore fetches
+  // chunk pos ^ lds_swz(r) of that row.
+  constexpr int kTileElems = BN * D;  // 8 KB per tile
+  __shared__ __align__(16) T Ksm[3][kTileElems];
+  __shared__ __align__(16) T Vsm[3][kTileElems];
+
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
+  const int nqt = (p.Lq + BM - 1) / BM;
+  int rank, bh;
+  xcd_tile_map(blockIdx.x, nqt, p.Hq * p.B, rank, bh);
+  const int qt = nqt - 1 - rank;
+  const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int q_row0 = qt * BM + w * (32 * RQ) + i32;
+
+  vec8 qf[RQ][DS];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_ld = min(q_row0 + 32 * a, p.Lq - 1);
+    const T* qp = q + b * p.q_stride[0] + h * p.q_stride[1] + (int64_t)q_ld * p.q_stride[2] + 8 * g;
+#pragma unroll
+    for (int s = 0; s < DS; s++) qf[a][s] = *reinterpret_cast<const vec8*>(qp + 16 * s);
+  }
+
+  // every key tile is visited and nothing is masked but (TAIL) the keys past the end: this kernel is
+  // launched for problems without tile lists and with a mask that hides nothing (mask code in the same
+  // function costs the unmasked path 3 %, hence the two instantiations)
+  const int nt = TAIL ? (p.Lkv + BN - 1) / BN : p.Lkv / BN;
+  auto tile_at = [&](int it) -> int { return it; };
+
+  const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
+  const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
+  const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
+
+  // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
+  const int fill_row = lane >> 3;                         // row inside the 8-row group
+  auto issue_tile = [&](int stage, int kv0) {
+    const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+      const int r0 = 16 * w + 8 * j;
+      const int fill_chunk = (lane & 7) ^ lds_swz<D>(8 * j + fill_row);  // logical chunk this lane fetches
+      const int row = min(r0 + fill_row, lim);
+      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + fill_chunk * 8;
+      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + fill_chunk * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
+    }
+  };
+  // ---- fragment reads ----
+  vec8 kfr[DS], vfr[2][DB], pf[2];
+  int koff[DS];  // element offsets of this lane's K row fragments inside a 32-row block
+#pragma unroll
+  for (int s = 0; s < DS; s++) koff[s] = i32 * D + (((2 * s + g) ^ lds_swz<D>(i32)) * 8);
+  auto read_k = [&](const T* Ks, int nb) {
+#pragma unroll
+    for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(Ks + nb * 32 * D + koff[s]);
+  };
+  // transposing reads: lane points at 4 elements of row 4g + (i16 >> 2) + 8e (+16tt), logical column
+  // 32db + 16h + 4(i16 & 3)
+  int voff[2][DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
+#pragma unroll
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        voff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
+      }
+  }
+  auto read_v = [&](const T* Vs, int nb) {
+#pragma unroll
+    for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const T* vp = Vs + (32 * nb + 16 * tt) * D;
+        vfr[tt][db] = join8<vec8>(lds_read_tr(vp + voff[0][db]), lds_read_tr(vp + voff[1][db]));
+      }
+  };
+
+  Score2<KIND> sm;
+  sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
+
+  float16_t oacc[RQ][DB], s_cur;
+  float m_run[RQ], l_run[RQ];
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    m_run[a] = -INFINITY;
+    l_run[a] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[a][db][r] = 0.f;
+  }
+  // nothing is pending before the first unit: P = 0 against V = 0
+#pragma unroll
+  for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+    for (int e = 0; e < 8; e++) pf[tt][e] = (T)0.f;
+#pragma unroll
+    for (int db = 0; db < DB; db++) vfr[tt][db] = pf[tt];
+  }
+
+  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  int t_cur = nt > 0 ? tile_at(0) : 0;
+  int t_nxt = nt > 1 ? tile_at(1) : 0;   // tile it + 1
+  int t_nx2 = nt > 2 ? tile_at(2) : 0;   // tile it + 2
+  if (nt > 0) issue_tile(0, t_cur * BN);
+  if (nt > 1) issue_tile(1, t_nxt * BN);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  // S of the first unit
+  read_k(Ksm[0], 0);
+#pragma unroll
+  for (int r = 0; r < 16; r++) s_cur[r] = 0.f;
+#pragma unroll
+  for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
+
+  const int slot = blockIdx.x >= (gridDim.x >> 1) ? 1 : 0;  // second half of the grid = second workgroup of a compute unit
+  int st = 0;  // LDS stage of the current tile (it % 3)
+  for (int it = 0; it < nt; it++) {
+    // Two workgroups share a compute unit and the instruction arbiter favours the older wave,
+    // which leaves the younger one behind until it runs alone at the end.  All workgroups have
+    // the same amount of work here, so trading the wave priority between them every tile keeps
+    // both advancing at the same pace.
+    if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
+    const int kv0 = t_cur * BN;
+    const int st_n = st == 2 ? 0 : st + 1;
+    const T* Ks = Ksm[st];
+    const T* Vs = Vsm[st];
+    const T* Kn = Ksm[st_n];
+    const int st_p = st == 0 ? 2 : st - 1;  // stage of the previous tile = stage of tile it + 2
+    const int kv_nx2 = t_nx2 * BN;
+    t_cur = t_nxt;
+    t_nxt = t_nx2;
+    if (it + 3 < nt) t_nx2 = tile_at(it + 3);
+#pragma unroll
+    for (int nb = 0; nb < 2; nb++) {
+#pragma unroll
+      for (int a = 0; a < RQ; a++) {
+        const int q_row = q_row0 + 32 * a;
+        if (nb == 1 && a == 0) {
+          // this wave's share of tile it + 1 has landed; after the barrier everyone's has, and
+          // the previous tile's stage (last read before this barrier) can take tile it + 2
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          __syncthreads();
+          if (it + 2 < nt) issue_tile(st_p, kv_nx2);
+        }
+        if (a == 1) read_v(Vs, nb);              // V columns of this step, first used in region B
+
+        // ---- region A: S^T of the next unit || score_mod relative to the running reference max ----
+        float16_t s_nxt;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s_nxt[r] = 0.f;
+#pragma unroll
+        for (int s = 0; s < DS; s++) s_nxt = Frag<T>::mfma(kfr[s], qf[1 - a][s], s_nxt);
+        const float m_use = (m_run[a] == -INFINITY) ? 0.f : m_run[a];
+        sm.tile(q_row, kv0 + nb * 32 + 4 * g);
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float s0 = s_cur[r], s1 = s_cur[r + 1];
+          if (ROUND_S) round_pair<T>(s0, s1);
+          s_cur[r] = sm.apply_sub(s0, acc_row(r), m_use);
+          s_cur[r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use);
+        }
+#pragma unroll
+        for (int i = 0; i < DS; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one matrix instruction
+          if (a == 1) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads (V columns)
+          __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);             // six vector instructions
+        }
+        if constexpr (TAIL) {
+          if (kv0 + BN > p.Lkv) {
+            // a real branch whose inputs pass through the asm, so that none of the mask
+            // arithmetic can be hoisted into the path of the complete tiles
+            int q_opaque = q_row, kv_opaque = kv0 + nb * 32;
+            asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
+            const int cls = band_block_class(p.mask, __builtin_amdgcn_readfirstlane(q_opaque - i32),
+                                             __builtin_amdgcn_readfirstlane(kv_opaque), 0x7fffffff, p.Lkv);
+            if (cls == kBlockNone) fill_masked(s_cur);
+            else if (cls == kBlockMixed) {
+              const Mask2 visible(p.mask, b, h, p.Lkv);
+              mask_block_q<false>(s_cur, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
+            }
+          }
+        }
+        // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
+        float m_rel = xhalf_max(block_max(s_cur));
+        const bool need = (m_rel > kTau) || (m_run[a] == -INFINITY && m_rel > -INFINITY);
+        if (__any(need)) {
+          asm volatile("" : "+v"(m_rel));  // keeps this rare path a real branch (never if-converted)
+          const float delta = need ? m_rel : 0.f;
+          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
+          m_run[a] = need ? (m_use + m_rel) : m_run[a];
+          l_run[a] *= alpha;
+#pragma unroll
+          for (int r = 0; r < 16; r++) s_cur[r] -= delta;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
+        }
+        // ---- region B: O^T += V^T.P^T of the previous unit || exponentials, rounding, row sum ----
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+          for (int db = 0; db < DB; db++) oacc[1 - a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[1 - a][db]);
+        vec8 pn[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+          typename Pair<T>::v2 pr[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const float p0 = fast_exp2(s_cur[8 * tt + 2 * e]);
+            const float p1 = fast_exp2(s_cur[8 * tt + 2 * e + 1]);
+            pr[e] = Pair<T>::pack(p0, p1);
+            l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+          }
+          pn[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        }
+        if (a == 0) read_k(nb == 0 ? Ks : Kn, nb == 0 ? 1 : 0);  // K rows of the next step (kfr is free after region A)
+#pragma unroll
+        for (int i = 0; i < 2 * DB; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // one matrix instruction
+          if (a == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read (K rows)
+          __builtin_amdgcn_sched_group_barrier(0x400, 4, 0);             // four exponentials
+          __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // rounding and row sum of the previous four
+        }
+        pf[0] = pn[0];
+        pf[1] = pn[1];
+        s_cur = s_nxt;
+      }
+    }
+    st = st_n;
+  }
+  __builtin_amdgcn_s_setprio(0);
+  // the last unit's P is still pending
+#pragma unroll
+  for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+    for (int db = 0; db < DB; db++) oacc[1][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[1][db]);
+
+  // ---- epilogue ----
+#pragma unroll
+  for (int a = 0; a < RQ; a++) {
+    const int q_row = q_row0 + 32 * a;
+    const float l_tot = xhalf_sum(l_run[a]);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (q_row < p.Lq) {
+      T* op = o + b * p.o_stride[0] + h * p.o_stride[1] + (int64_t)q_row * p.o_stride[2] + 4 * g;
+#pragma unroll
+      for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int rr = 0; rr < 4; rr++) {
+          union { T e[4]; uint2 u; } pk;
+#pragma unroll
+          for (int e = 0; e < 4; e++) pk.e[e] = (T)(oacc[a][db][4 * rr + e] * inv);
+          *reinterpret_cast<uint2*>(op + 32 * db + 8 * rr) = pk.u;
+        }
+      if (lse2 && g == 0) lse2[((int64_t)b * p.Hq + h) * p.Lq + q_row] = l_tot > 0.f ? m_run[a] + log2f(l_tot) : -INFINITY;
+    }
+  }
+}
+
+struct FwdArgs {
+  const void *q, *k, *v;
+  void* o;
+  float* lse2;
+  hipStream_t s;
+};
+
+template <typename T, int D, int KIND, bool RS, bool BITS, int PASS>
+static void launch_list_kernel(const FlexAttnParams& p, const FwdArgs& a) {
+  dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B);
+  hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, RS, BITS, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
+                     (const T*)a.v, (T*)a.o, a.lse2);
+}
+
+template <typename T, int KIND, bool RS, bool TAIL>
+static void launch_pipe_kernel(const FlexAttnParams& p, const FwdArgs& a) {
+  dim3 grid((p.Lq + kPipeBM - 1) / kPipeBM * p.Hq * p.B);
+  hipLaunchKernelGGL((fwd_pipe_kernel<T, KIND, RS, TAIL>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k, (const T*)a.v,
+                     (T*)a.o, a.lse2);
+}
+
+template <typename T, int D, int KIND>
+static void launch_rs(const FlexAttnParams& p, const FwdArgs& a) {
+  const bool bits = p.mask.kind == FLEX_MASK_BITS;
+  if (p.flags & FLEX_PARITY) {
+    // parity numerics: a log-sum-exp pass, then the pass that multiplies the normalised, rounded P into V
+    // (a.lse2 is never null here: the caller substitutes workspace); S is always rounded through the input dtype
+    if (bits) {
+      launch_list_kernel<T, D, KIND, true, true, kFwdLse>(p, a);
+      launch_list_kernel<T, D, KIND, true, true, kFwdNorm>(p, a);
+    } else {
+      launch_list_kernel<T, D, KIND, true, false, kFwdLse>(p, a);
+      launch_list_kernel<T, D, KIND, true, false, kFwdNorm>(p, a);
+    }
+    return;
+  }
+  // D = 64 without tile lists or anything to mask (every workgroup has the same work): the pipelined
+  // kernel with 256-row workgroups.  Otherwise the 128-row kernel: twice the workgroups, half the length of the
+  // longest one, which is what bounds a causal-like schedule.
+  // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
+  if constexpr (KIND != FLEX_SCORE_AFFINE && D == 64) {
+    if (!p.tiles.kv_num && mask_hides_nothing(p.mask)) {
+      const bool tail = p.Lkv % kFwdBN != 0, rs = (p.flags & FLEX_ROUND_S) != 0;
+      if (rs && !tail) launch_pipe_kernel<T, KIND, true, false>(p, a);
+      else if (rs) launch_pipe_kernel<T, KIND, true, true>(p, a);
+      else if (!tail) launch_pipe_kernel<T, KIND, false, false>(p, a);
+      else launch_pipe_kernel<T, KIND, false, true>(p, a);
+      return;
+    }
+  }
+  if (p.flags & FLEX_ROUND_S) {
+    if (bits) launch_list_kernel<T, D, KIND, true, true, kFwdOnePass>(p, a);
+    else launch_list_kernel<T, D, KIND, true, false, kFwdOnePass>(p, a);
+  } else {
+    if (bits) launch_list_kernel<T, D, KIND, false, true, kFwdOnePass>(p, a);
+    else launch_list_kernel<T, D, KIND, false, false, kFwdOnePass>(p, a);
+  }
+}
+
+template <typename T, int D>
+static int launch_kind(const FlexAttnParams& p, const FwdArgs& a) {
+  switch (p.score.kind) {
+    case FLEX_SCORE_IDENTITY: launch_rs<T, D, FLEX_SCORE_IDENTITY>(p, a); return 0;
+    case FLEX_SCORE_CHECKERBOARD: launch_rs<T, D, FLEX_SCORE_CHECKERBOARD>(p, a); return 0;
+    case FLEX_SCORE_ALIBI: launch_rs<T, D, FLEX_SCORE_ALIBI>(p, a); return 0;
+    case FLEX_SCORE_TANH_SOFTCAP: launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, a); return 0;
+    case FLEX_SCORE_REL_BIAS: launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, a); return 0;
+    case FLEX_SCORE_AFFINE: launch_rs<T, D, FLEX_SCORE_AFFINE>(p, a); return 0;
+  }
+  return 1;
+}
+
+}  // namespace flex

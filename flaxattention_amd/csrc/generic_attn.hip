@@ -223,7 +223,9 @@ __global__ __launch_bounds__(kWaves * 64) void generic_dq_kernel(FlexAttnParams 
     if (strict) dp = round_through<T>(dp);
     dsum += pr * dp;
   }
-  const float dl = wave_sum(dsum);
+  float dl = wave_sum(dsum);
+  // cotangent of the log-sum-exp output: d lse / d X_ij = P_ij joins the row term
+  if (p.d_lse2 && row_ok) dl -= kLog2e * p.d_lse2[row_id];
   if (row_ok && lane == 0) delta[row_id] = dl;
 
   float acc[kMaxAcc];

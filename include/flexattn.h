@@ -95,6 +95,15 @@ enum FlexFlags {
                             dP and dS through the input dtype (attention.py:105
                             and its transposes) */
   FLEX_FORCE_GENERIC = 4, /* never use the MFMA kernels */
+  FLEX_PARITY = 32,      /* fused (MFMA) kernels with the rounding points of the reference's dense
+                            path (attention.py:27, 104-105 and their transposes under jax.grad):
+                            forward in two passes (log-sum-exp, then the NORMALISED P rounded to
+                            the input dtype and multiplied into V); backward with dP rounded to the
+                            input dtype, delta_i = sum_j P_ij round(dP_ij) from a row sweep of its
+                            own, and the scale applied before dS is rounded.  Implies FLEX_ROUND_S.
+                            Costs about 1.5x the time of the default numerics, which round the
+                            unnormalised P and use delta = sum_d O dO.  Where only the generic
+                            kernels apply the flag means FLEX_STRICT.  */
   /* profiling aids for flexattn_bwd: launch only one of the two fused backward
    * kernels.  The dK/dV kernel then reads the delta values a previous complete
    * call left in the same workspace. */
@@ -141,6 +150,10 @@ typedef struct FlexAttnParams {
    * against a long KV cache as several decode calls.  A multiple of 64. */
   int32_t q_index_base;
   int32_t pad_;
+  /* flexattn_bwd only, optional (NULL = zero): cotangent of the lse2 output, [B,Hq,Lq] fp32.
+   * In the reference the log-sum-exp is an ordinary differentiable output of math_attention
+   * (attention.py:97-106); d lse / d score_ij = P_ij joins the softmax's row term.  */
+  const float* d_lse2;
 } FlexAttnParams;
 
 int flexattn_abi_version(void);
@@ -171,7 +184,9 @@ int flexattn_block_mask_build(const FlexMask* mask, int32_t B, int32_t H,
                               int32_t* full_q_num, int32_t* full_q_idx,
                               void* workspace, flexattn_stream_t stream);
 
-/* Forward.  Replaces math_attention (flaxattention/core/attention.py:67-106)
+/* Forward.  With FLEX_PARITY and lse2 == NULL the log-sum-exp that the second pass reads is kept
+ * in `workspace` (flexattn_fwd_workspace_bytes); otherwise workspace may be NULL.
+ * Replaces math_attention (flaxattention/core/attention.py:67-106)
  * behind flax_attention (169-218) and mha_forward_kernel / _mha_forward
  * (flaxattention/kernel/attention.py:34-149, 260-335) behind
  * flax_attention_pallas (attention.py:220-312).  o: same layout family as q
@@ -184,7 +199,8 @@ int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const vo
 /* Backward.  Replaces jax.grad through math_attention (the reference's pure
  * path) and _preprocess_backward / mha_backward_kernel / _mha_backward
  * (flaxattention/kernel/attention.py:338-650).  P is recomputed from lse2.
- * dq/dk/dv are contiguous [B,H,L,D] tensors of the input dtype.  */
+ * d_o is a contiguous [B,Hq,Lq,Dv] tensor (the strides in `p` describe q, k,
+ * v and o only); dq/dk/dv are contiguous [B,H,L,D] tensors of the input dtype.  */
 size_t flexattn_bwd_workspace_bytes(const FlexAttnParams* p);
 int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* k, const void* v,
                  const void* o, const float* lse2, const void* d_o,
@@ -211,28 +227,6 @@ int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const
 #define FLEXATTN_DECODE_STATIC_BYTES ((size_t)16 << 20)
 int flexattn_decode_static(const FlexAttnParams* p, const void* q, const void* k, const void* v,
                            void* o, float* lse2, int32_t num_splits, flexattn_stream_t stream);
-
-/* Measurement aid with no counterpart in the reference: launches a kernel that only
- * issues v_mfma_f32_32x32x16_f16 on pseudo-random operands (512 workgroups x 4 waves,
- * 8*iters MFMAs per wave) so that a caller can time the matrix throughput the GPU
- * sustains under its power limit.  `sink` is a device buffer of 512*256 floats;
- * *flops_per_launch receives the flop count of one launch. */
-int flexattn_probe_mfma(float* sink, int32_t iters, double* flops_per_launch, flexattn_stream_t stream);
-
-/* Second measurement aid, also without counterpart in the reference: the instruction mix of a
- * fused attention step.  Per unit a wave issues `mfma_per_unit` (8, 12 or 16) matrix
- * instructions interleaved with 80 fused multiply-adds and 16 exponentials (the vector work of
- * one 32x32 score block), two waves per SIMD, `iters` units per wave.  Its matrix flop rate is
- * the ceiling of that mix on this GPU (matrix and vector instructions share the issue port and
- * the power budget): 8 = forward at D 64, 12 = dQ kernel, 16 = dK/dV kernel or forward at D 128.
- * `sink` as above; *flops_per_launch receives the matrix flop count of one launch. */
-int flexattn_probe_mix(float* sink, int32_t iters, int32_t mfma_per_unit, double* flops_per_launch,
-                       flexattn_stream_t stream);
-
-/* Third measurement aid without counterpart in the reference: a kernel that only reads `bytes` of device memory
- * (16-byte loads, 1024 workgroups), for the read rate that memory delivers to a kernel that does nothing else; the
- * decode kernel is held against it.  `sink`: 65536 floats, practically never written. */
-int flexattn_probe_read(const void* src, size_t bytes, float* sink, flexattn_stream_t stream);
 
 #ifdef __cplusplus
 }

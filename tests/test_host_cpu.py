@@ -163,6 +163,16 @@ def test_untagged_score_mods_are_recognised():
     assert resolve_score_mod(lambda s, b, h, q, kv: s, 4).kind == _lib.SCORE_IDENTITY
     assert resolve_score_mod(None, 4).kind == _lib.SCORE_IDENTITY
     assert _probe_score_mod(lambda s, b, h, q, kv: s * s, 4) is None
+    # mods that equal a family near the origin only: the family must not be accepted for them
+    far = lambda s, b, h, q, kv: torch.where((q - kv).abs() > 64, s - 10.0, s)          # noqa: E731
+    late_batch = lambda s, b, h, q, kv: torch.where(b >= 2, s * 0.5, s)                  # noqa: E731
+    segments = lambda s, b, h, q, kv: s + ((q // 16) != (kv // 16)) * -5.0               # noqa: E731
+    for fn in (far, late_batch, segments):
+        assert _probe_score_mod(fn, 4, (4, 4, 256, 256)) is None, fn
+        assert _probe_score_mod(fn, 4) is None, fn
+    # ... while on a problem that never leaves the region where they agree, the family is the right lowering
+    assert _probe_score_mod(late_batch, 4, (2, 4, 64, 64)).kind == _lib.SCORE_IDENTITY
+    assert _probe_score_mod(far, 4, (1, 4, 32, 32)).kind == _lib.SCORE_IDENTITY
     with pytest.raises(NotImplementedError):
         resolve_score_mod(lambda s, b, h, q, kv: torch.sin(s), 4)
 
