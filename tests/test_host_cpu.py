@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in decl:
         assert hasattr(L, name), name
-    assert L.flexattn_abi_version() == 2
+    assert L.flexattn_abi_version() == 3
     assert L.flexattn_last_error() is not None
 
 
