@@ -7,8 +7,19 @@ A "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM.  The default workload is benchmark configuration 2
 (fp16 [8,8,2048,64], checkerboard score_mod, no mask, forward + backward of
 out.sum()); one step = forward kernel + both backward kernels.  The last line
-printed on stdout is ONE JSON object (the driver's contract); --all prints
-per-configuration lines to stderr first.
+printed on stdout is ONE JSON object (the driver's contract).  Besides the
+headline it carries the decode half of the metric (configuration 5, q_len 1,
+16 and 64 over rotating KV caches: us, GB/s, fraction of 8 TB/s), the step
+times of configurations 3 and 4, and every training configuration in both
+numerics modes ("fast" and "parity"); --all adds the probes, the split sweep
+of the decode kernel and the block-mask builder.
+
+Kernel durations are HIP-event intervals taken INSIDE the step (forward, dQ
+and dK/dV launched in their real order, an event between them): a kernel
+timed in a loop of its own runs 6-7 % faster than inside the step, where the
+previous kernel has left other data in the caches.  rocprofv3 --kernel-trace
+of this same command shows the same durations and no gaps between the three
+kernels, so step time = sum of kernel times.
 
 Throughput counts algorithmic flops only: 4*bq*bk*D per visible tile in the
 forward and 10*bq*bk*D in the backward at the 128x128 granularity of the block
@@ -32,9 +43,11 @@ PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 PEAK_HBM_GBPS = 8000.0
 
 
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE from two `rocprofv3 --pmc` runs of `bench.py --pmc-probe`, each
-# counter scaled by what it reads for a 1 GiB device copy: x2.000 and x1.000); the summary of those runs is kept
-# under profiles/.  Keyed by (workload, kernel); a kernel that has not been measured reports null.
+# HBM bytes per launch.  A timing run cannot read hardware counters, so these are copied from the counter runs
+# summarised in TRAFFIC_SOURCE (two `rocprofv3 --pmc` runs of `python3 bench.py --pmc-probe`, FETCH_SIZE then
+# WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB device copy at the start of that run).
+# Keyed by (workload, kernel); a kernel that has not been measured reports null.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_config2_and_decode_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
     ("config2", "fwd_pipe_kernel"): 67791802,
     ("config2", "bwd_dq_kernel"): 136751025,
@@ -56,8 +69,9 @@ class Prepared:
         from flaxattention_amd.core.attention import _make_plan
         self.L = _lib.lib()
         self._lib = _lib
-        g = torch.Generator(device="cpu").manual_seed(seed)
-        mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32).to(dtype).to(dev)
+        # standard normal, drawn on the device (seeded): nothing in a measurement waits for the host to make data
+        g = torch.Generator(device=dev).manual_seed(seed)
+        mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32, device=dev).to(dtype)
         self.k, self.q, self.v = mk(B, Hkv, Lkv, D), mk(B, Hq, Lq, D), mk(B, Hkv, Lkv, D)
         self.d_o = torch.ones(B, Hq, Lq, D, dtype=dtype, device=dev)   # gradient of out.sum()
         bm = fa.create_block_mask(mask, 1, 1, Lq, Lkv, device=dev) if mask is not None else None
@@ -123,6 +137,33 @@ def event_time_us(fn, n, warm=3):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e3 / n
+
+
+def step_kernel_times_us(pr, n, warm=3):
+    """Durations of the three C calls of a training step, each measured inside the step: forward, dQ (in the parity
+    numerics: the row sweep for delta + dQ) and dK/dV are launched in their real order with a HIP event between
+    them.  Median over n steps."""
+    def one(ev):
+        ev[0].record()
+        pr.fwd()
+        ev[1].record()
+        pr.bwd("dq")
+        ev[2].record()
+        pr.bwd("dkv")
+        ev[3].record()
+    scratch = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    for _ in range(warm):
+        one(scratch)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n)]
+    torch.cuda.synchronize()
+    for ev in evs:
+        one(ev)
+    torch.cuda.synchronize()
+    out = []
+    for j in range(3):
+        d = sorted(ev[j].elapsed_time(ev[j + 1]) * 1e3 for ev in evs)
+        out.append(d[len(d) // 2])
+    return out
 
 
 def wall_time_ms(fn, steps, warmup):
@@ -205,16 +246,20 @@ def run_train_config(dev, name, steps, warmup, opts=None, graph=False):
     else:
         ms = wall_time_ms(step, steps, warmup)
     n = max(steps, 10)
-    # D = 64: the pipelined kernel runs when there are no tile lists, the list-driven kernel otherwise
-    fwd_name = "fwd_pipe_kernel" if pr.block_mask is None else "fwd_mfma_kernel"
-    us = {fwd_name: event_time_us(pr.fwd, n),
-          "bwd_dq_kernel": event_time_us(lambda: pr.bwd("dq"), n),
-          "bwd_dkv_kernel": event_time_us(lambda: pr.bwd("dkv"), n)}
-    alg = {fwd_name: f_fwd, "bwd_dq_kernel": 2 * per_tile * tiles, "bwd_dkv_kernel": 8 * per_tile * tiles}
-    kern = {k: {"us": round(us[k], 2), "algorithmic_flops": alg[k], "tflops": round(alg[k] / us[k] / 1e6, 1)} for k in us}
+    parity = bool(pr.p.flags & pr._lib.FLAG_PARITY)
+    # D = 64: the pipelined kernel runs when there are no tile lists and the numerics are "fast", the list-driven
+    # kernel otherwise (twice in the parity numerics: log-sum-exp pass, then the normalised pass)
+    fwd_name = "fwd_pipe_kernel" if (pr.block_mask is None and not parity) else "fwd_mfma_kernel"
+    dq_name = "bwd_dq_kernel" if not parity else "bwd_dq_kernel (row sweep for delta + dQ)"
+    t = step_kernel_times_us(pr, n)
+    us = {fwd_name: t[0], dq_name: t[1], "bwd_dkv_kernel": t[2]}
+    alg = {fwd_name: f_fwd, dq_name: 2 * per_tile * tiles, "bwd_dkv_kernel": 8 * per_tile * tiles}
+    kern = {k: {"us": round(us[k], 2), "algorithmic_flops": alg[k], "tflops": round(alg[k] / us[k] / 1e6, 1),
+                "frac_mfma_peak": round(alg[k] / us[k] / 1e6 / PEAK_MFMA_TFLOPS, 4)} for k in us}
     dom = max(us, key=us.get)
     return {"ms_per_step": ms, "tflops": (f_fwd + f_bwd) / ms / 1e9, "fwd_tflops": f_fwd / us[fwd_name] / 1e6,
-            "bwd_tflops": f_bwd / (us["bwd_dq_kernel"] + us["bwd_dkv_kernel"]) / 1e6,
+            "bwd_tflops": f_bwd / (us[dq_name] + us["bwd_dkv_kernel"]) / 1e6,
+            "kernel_sum_us": sum(us.values()),
             "kernels": kern, "dominant": dom, "dtype": dtype, "flops": f_fwd + f_bwd}
 
 
@@ -300,9 +345,11 @@ def run_mix_probe(dev):
 
 
 def run_read_probe(dev):
-    """Read rate of the bare streaming-read kernel over 268 MB (the K + V bytes of one decode call of
-    configuration 5): rotating over three buffers, which no launch finds in the 256 MB last-level cache, and
-    re-reading one buffer.  GB/s."""
+    """Read rate of the bare streaming-read kernel, GB/s.  (a) 268 MB (the K + V bytes of one decode call of
+    configuration 5) rotating over three buffers, which no launch finds in the 256 MB last-level cache, and
+    re-reading one buffer; (b) the same kernel over 2 GiB at several grid sizes and loads in flight per thread: at
+    that size launch ramp and tail are under 2 % of the run, so the best of these is the steady-state read rate of
+    the memory system, against which the 268 MB figure shows what a 50 us kernel loses to ramp and tail."""
     L = probe_lib()
     nbytes = 2 * 8 * 8 * 16384 * 64 * 2
     bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(3)]
@@ -310,13 +357,27 @@ def run_read_probe(dev):
     stream = torch.cuda.current_stream(dev).cuda_stream
     turn = [0]
 
-    def go(n_bufs):
-        rc = L.flexprobe_read(bufs[turn[0] % n_bufs].data_ptr(), nbytes, sink.data_ptr(), 0, 0, stream)
+    def go(n_bufs, wgs=0, nld=0):
+        rc = L.flexprobe_read(bufs[turn[0] % n_bufs].data_ptr(), nbytes, sink.data_ptr(), wgs, nld, stream)
         turn[0] += 1
         probe_check(rc, "flexprobe_read")
-    cold = event_time_us(lambda: go(3), 30)
-    warm = event_time_us(lambda: go(1), 30)
-    return {"rotating_buffers": round(nbytes / cold / 1e3), "one_buffer": round(nbytes / warm / 1e3)}
+    out = {"rotating_buffers": round(nbytes / event_time_us(lambda: go(3), 30) / 1e3),
+           "one_buffer": round(nbytes / event_time_us(lambda: go(1), 30) / 1e3)}
+    shapes = {}
+    for wgs in (512, 1024, 2048, 4096, 8192):
+        for nld in (2, 4, 8, 16):
+            shapes[f"{wgs}x{nld}"] = round(nbytes / event_time_us(lambda: go(3, wgs, nld), 15) / 1e3)
+    out["rotating_268MB_by_workgroups_x_loads"] = shapes
+    del bufs
+    big = torch.randint(0, 255, (2 << 30,), dtype=torch.uint8, device=dev)
+    steady = {}
+    for wgs in (1024, 2048, 4096, 8192):
+        for nld in (4, 8, 16):
+            def one():
+                probe_check(L.flexprobe_read(big.data_ptr(), big.numel(), sink.data_ptr(), wgs, nld, stream), "flexprobe_read")
+            steady[f"{wgs}x{nld}"] = round(big.numel() / event_time_us(one, 5, warm=1) / 1e3)
+    out["steady_2GiB_by_workgroups_x_loads"] = steady
+    return out
 
 
 def run_block_mask_build(dev):
@@ -332,11 +393,11 @@ def run_block_mask_build(dev):
     return out
 
 
-def run_config4(dev, steps, warmup):
+def run_config4(dev, steps, warmup, opts=None):
     from flaxattention_amd.masks import generate_attention_sink
     from flaxattention_amd.mods import generate_tanh_softcap
     # |q-kv| <= 1024 causal window, kv < 4 always visible, tanh soft-cap 50
-    pr = Prepared(dev, torch.bfloat16, 4, 16, 16, 8192, 8192, 128, generate_tanh_softcap(50.0), generate_attention_sink(1024, 3))
+    pr = Prepared(dev, torch.bfloat16, 4, 16, 16, 8192, 8192, 128, generate_tanh_softcap(50.0), generate_attention_sink(1024, 3), opts)
     bm = pr.block_mask
     tiles = int(bm.kv_num_blocks.sum().item() + bm.full_kv_num_blocks.sum().item()) * 4 * 16
     flops = 4 * 128 * 128 * 128 * tiles
@@ -357,7 +418,7 @@ def run_config5(dev, steps, warmup, sweep=True):
     for ql in (1, 16, 64):
         byts = 2 * 8 * 8 * Lkv * 64 * 2 + 2 * 8 * 8 * ql * 64 * 2
         best = None
-        for splits in ((8, 12, 16) if sweep else (12,)):
+        for splits in ((8, 12, 16) if sweep else (8,)):
             prs = [Prepared(dev, torch.float16, 8, 8, 8, ql, Lkv, 64, generate_alibi_bias(8, -1.0), offset_causal_mask(Lkv - ql),
                             decode_splits=splits, seed=s) for s in range(n_sets)]
             turn = [0]
@@ -376,6 +437,12 @@ def run_config5(dev, steps, warmup, sweep=True):
     return out
 
 
+def mode_summary(r):
+    return {"ms_per_step": round(r["ms_per_step"], 4), "fwd_bwd_tflops": round(r["tflops"], 1),
+            "pct_mfma_peak": round(r["tflops"] / PEAK_MFMA_TFLOPS * 100, 2),
+            "kernels_us": {k: v["us"] for k, v in r["kernels"].items()}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -383,8 +450,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="config2", choices=["config2", "config3"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--all", action="store_true", help="also run configurations 3, 4 and 5 (reported on stderr and in 'extra')")
+    ap.add_argument("--headline-only", action="store_true", help="only the headline workload (no other configurations, modes or decode)")
+    ap.add_argument("--all", action="store_true", help="also the probes, the decode split sweep and the block-mask builder (in 'extra')")
     ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
+    ap.add_argument("--numerics", default=None, choices=["fast", "parity"],
+                    help="numerics of the headline workload (default: the library's: fp16 fast, bf16 parity)")
     ap.add_argument("--graph", action="store_true", help="replay the three kernels of a step as one HIP graph instead of launching them eagerly")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter run: one 1 GiB device copy (calibration) and 3 launches of each kernel of the workload, nothing else")
@@ -398,18 +468,54 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda", 0)
     opts = {"round_s": bool(a.round_s)}
+    if a.numerics:
+        opts["numerics"] = a.numerics
     if a.pmc_probe:
         pmc_probe(dev, a.workload, opts)
         return
+    line_extra = {}
+    if not a.headline_only:
+        # order: the bandwidth-bound decode first, the headline's own kernels last
+        c5 = run_config5(dev, a.steps, a.warmup, sweep=a.all)
+        for ql, d in c5.items():
+            log(f"config5 q_len {ql}: decode {d['decode_us']:.1f} us over rotating KV caches ({d['decode_gbps']:.0f} GB/s, "
+                f"{d['decode_gbps'] / PEAK_HBM_GBPS * 100:.1f}% of HBM peak, {d['splits']} splits; {d['decode_us_same_cache']:.1f} us when one "
+                f"cache is re-read); prefill kernel {d['prefill_kernel_us']:.1f} us")
+        d1 = c5[1]
+        line_extra["decode"] = {
+            "workload": "configs[4]: fp16 Q [8,8,q_len,64] against KV [8,8,16384,64], ALiBi, offset-causal; calls rotate over "
+                        "three KV caches (805 MB) so that none is served from the 256 MB last-level cache",
+            "us": round(d1["decode_us"], 1), "gbps": round(d1["decode_gbps"]), "bytes": d1["bytes"],
+            "frac_hbm_peak": round(d1["decode_gbps"] / PEAK_HBM_GBPS, 3), "peak_gbps": PEAK_HBM_GBPS,
+            "by_q_len": {str(ql): {"us": round(d["decode_us"], 1), "gbps": round(d["decode_gbps"]), "bytes": d["bytes"],
+                                   "frac_hbm_peak": round(d["decode_gbps"] / PEAK_HBM_GBPS, 3), "splits": d["splits"],
+                                   "us_same_cache": round(d["decode_us_same_cache"], 1),
+                                   "prefill_kernel_us": round(d["prefill_kernel_us"], 1)} for ql, d in c5.items()}}
+        # every training configuration in both numerics modes
+        c4 = {}
+        for num in ("parity", "fast"):
+            x = run_config4(dev, a.steps, a.warmup, dict(opts, numerics=num))
+            c4[num] = {"fwd_us": round(x["us"], 1), "fwd_tflops": round(x["tflops"], 1),
+                       "pct_mfma_peak": round(x["tflops"] / PEAK_MFMA_TFLOPS * 100, 2), "default": num == "parity"}
+            log(f"config4 numerics {num}: fwd {x['us']:.1f} us  {x['tflops']:.1f} TFLOP/s on {x['tiles_per_head']} tiles/head")
+        modes = {}
+        for wl, default in (("config3", "parity"), ("config2", "fast")):
+            modes[wl] = {}
+            for num in ("parity", "fast"):
+                rr = run_train_config(dev, wl, a.steps, a.warmup, dict(opts, numerics=num))
+                modes[wl][num] = mode_summary(rr)
+                modes[wl][num]["default"] = num == default
+                log(f"{wl} numerics {num}: {rr['ms_per_step'] * 1e3:.1f} us/step  {rr['tflops']:.1f} TFLOP/s  {modes[wl][num]['kernels_us']}")
+        modes["config4"] = c4
+        line_extra["numerics_modes"] = modes
+    # The headline comes last: by now the GPU has been under load for seconds.  Started from idle, the first ~50
+    # steps (20 ms) run through a transient of the power management (step times of 370 -> 530 -> 360 us in a kernel
+    # trace); W warm-up steps and K timed steps placed there would measure that transient, not the sustained rate.
     r = run_train_config(dev, a.workload, a.steps, a.warmup, opts, graph=a.graph)
-    log(f"{a.workload}: {r['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r['tflops']:.1f} TFLOP/s  "
+    log(f"{a.workload}: {r['ms_per_step'] * 1e3:.1f} us/step (kernel sum {r['kernel_sum_us']:.1f} us)  fwd+bwd {r['tflops']:.1f} TFLOP/s  "
         f"(fwd {r['fwd_tflops']:.1f}, bwd {r['bwd_tflops']:.1f})  kernels {r['kernels']}")
     extra = {}
     if a.all:
-        other = "config3" if a.workload == "config2" else "config2"
-        r2 = run_train_config(dev, other, a.steps, a.warmup, opts, graph=a.graph)
-        log(f"{other}: {r2['ms_per_step'] * 1e3:.1f} us/step  fwd+bwd {r2['tflops']:.1f} TFLOP/s  kernels {r2['kernels']}")
-        extra[other] = {"ms_per_step": round(r2["ms_per_step"], 4), "fwd_bwd_tflops": round(r2["tflops"], 1), "kernels": r2["kernels"]}
         probe = run_mfma_probe(dev)
         log(f"MFMA-only probe kernel (fp16, pseudo-random operands): {probe:.0f} TFLOP/s sustained")
         extra["mfma_probe_tflops"] = round(probe, 1)
@@ -417,40 +523,37 @@ def main():
         log(f"instruction-mix probe (MFMAs per 96 vector instructions -> matrix TFLOP/s): {mix}")
         extra["mix_probe_tflops"] = mix
         rd = run_read_probe(dev)
-        log(f"bare read of 268 MB: {rd['rotating_buffers']} GB/s over rotating buffers, {rd['one_buffer']} GB/s re-reading one buffer")
+        log(f"bare read: {rd}")
         extra["read_probe_gbps"] = rd
         bmb = run_block_mask_build(dev)
         log(f"create_block_mask: {bmb} us")
         extra["block_mask_build_us"] = bmb
-        c4 = run_config4(dev, a.steps, a.warmup)
-        log(f"config4: fwd {c4['us']:.1f} us  {c4['tflops']:.1f} TFLOP/s on {c4['tiles_per_head']} tiles/head")
-        extra["config4"] = {"fwd_us": round(c4["us"], 1), "fwd_tflops": round(c4["tflops"], 1)}
-        c5 = run_config5(dev, a.steps, a.warmup)
-        for ql, d in c5.items():
-            log(f"config5 q_len {ql}: decode {d['decode_us']:.1f} us over rotating KV caches ({d['decode_gbps']:.0f} GB/s, "
-                f"{d['decode_gbps'] / PEAK_HBM_GBPS * 100:.1f}% of HBM peak, {d['splits']} splits; {d['decode_us_same_cache']:.1f} us when one "
-                f"cache is re-read); prefill kernel {d['prefill_kernel_us']:.1f} us")
-        extra["config5"] = {str(ql): {"decode_us": round(d["decode_us"], 1), "decode_gbps": round(d["decode_gbps"]),
-                                      "frac_hbm_peak": round(d["decode_gbps"] / PEAK_HBM_GBPS, 3), "splits": d["splits"],
-                                      "decode_us_same_cache": round(d["decode_us_same_cache"], 1),
-                                      "prefill_kernel_us": round(d["prefill_kernel_us"], 1)} for ql, d in c5.items()}
     dom = r["dominant"]
     kd = r["kernels"][dom]
     line = {
-        "metric": "fwd+bwd TFLOP/s (B8 H8 L2048 D64, algorithmic flops of unmasked 128x128 tiles)",
+        "metric": "fwd+bwd TFLOP/s (B8 H8 L2048 D64, algorithmic flops of unmasked 128x128 tiles); decode HBM GB/s in 'decode'",
         "value": round(r["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(r["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": r["dtype"], "data": "synthetic",
         "config": {"workload": {"config2": "configs[1]: fp16 [8,8,2048,64] checkerboard score_mod, no mask, forward + backward of out.sum()",
                                 "config3": "configs[2]: bf16 [8,8,2048,64] ALiBi score_mod, causal block mask 128x128, forward + backward of out.sum()"}[a.workload],
-                   "round_s": bool(a.round_s), "launch": "hip graph replay" if a.graph else "eager"},
+                   "round_s": bool(a.round_s), "numerics": a.numerics or ("fast" if a.workload == "config2" else "parity"),
+                   "launch": "hip graph replay" if a.graph else "eager"},
         "pct_mfma_peak": round(r["tflops"] / PEAK_MFMA_TFLOPS * 100, 2),
         "fwd_tflops": round(r["fwd_tflops"], 1), "bwd_tflops": round(r["bwd_tflops"], 1),
+        "kernel_sum_us": round(r["kernel_sum_us"], 1),
         "kernels": r["kernels"],
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": kd["tflops"], "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kd["tflops"] / PEAK_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom))},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom)), "traffic_source": TRAFFIC_SOURCE,
+                     "duration_source": "HIP events around the kernel inside the step (median); rocprofv3 --kernel-trace of "
+                                        "this command agrees (profiles/fwd_bwd_config2_kernel_trace.md)",
+                     "attribution": "S and dP are computed by both backward kernels; they are attributed to bwd_dkv_kernel "
+                                    "(8 of the convention's 10 backward units), dQ alone to bwd_dq_kernel",
+                     "frac_by_kernel": {k: v["frac_mfma_peak"] for k, v in r["kernels"].items()},
+                     "frac_whole_step": round(r["tflops"] / PEAK_MFMA_TFLOPS, 4)},
     }
+    line.update(line_extra)
     if extra:
         line["extra"] = extra
     if not a.no_cpu:
