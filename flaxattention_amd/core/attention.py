@@ -271,6 +271,7 @@ def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o, d_lse2=None) -> Tuple[Array, Ar
     dq = torch.empty((plan.B, plan.Hq, plan.Lq, plan.D), dtype=q.dtype, device=q.device)
     dk = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.D), dtype=q.dtype, device=q.device)
     dv = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.Dv), dtype=q.dtype, device=q.device)
+    plan.mask.ensure_transposed()   # the dK/dV kernel reads a bitmap mask packed along the query axis
     p = plan.params(q, k, v, o)
     p.d_lse2 = d_lse2.data_ptr() if d_lse2 is not None else None
     with torch.cuda.device(q.device):

@@ -356,6 +356,23 @@ class MaskMod:
     def is_noop(self) -> bool:
         return self.bits is None and self.lo == INT_MIN and self.hi == INT_MAX
 
+    def ensure_transposed(self) -> None:
+        """Make the query-packed copy of a bitmap (what the dK/dV kernel reads) if it does not exist yet: large
+        bitmaps are lowered without it, so that a forward-only user never holds the second copy.  Built from the
+        key-packed words on the device, one (batch, head) slab of rows at a time."""
+        if self.bits is None or self.bits_t is not None:
+            return
+        Bm, Hm, Qp, W = self.bits.shape
+        KVp = W * 32
+        out = torch.empty((Bm, Hm, KVp, Qp // 32), dtype=torch.int32, device=self.bits.device)
+        rows = max(32, min(Qp, (_SLAB_ELEMS // KVp) // 32 * 32))
+        for b in range(Bm):
+            for h in range(Hm):
+                for q0 in range(0, Qp, rows):
+                    m = unpack_bits(self.bits[b, h, q0:q0 + rows], KVp)          # [rows, KVp]
+                    out[b, h, :, q0 // 32:(q0 + m.shape[0]) // 32] = pack_bits(m.transpose(0, 1).contiguous())
+        self.bits_t = out
+
     def key(self):
         if self.bits is not None:
             return ("bits", self.bits.data_ptr())
@@ -530,7 +547,8 @@ def _stamp_valid(stamp, now=None) -> bool:
 
 
 def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device,
-                         real: Optional[Tuple[int, int]] = None) -> torch.Tensor:
+                         real: Optional[Tuple[int, int]] = None, b_range: Optional[Tuple[int, int]] = None,
+                         h_range: Optional[Tuple[int, int]] = None, q_range: Optional[Tuple[int, int]] = None) -> torch.Tensor:
     """Evaluate a Python mask_mod (or a five-argument score_mod) over the index grid [0,Q) x [0,KV) with
     device tensors.  bool, broadcastable to [B,H,Q,KV].
 
@@ -540,17 +558,36 @@ def dense_mask_on_device(fn: Callable, B: int, H: int, Q: int, KV: int, device,
     the process, and torch accepts CPU index tensors for device tensors, so trying on the CPU first is no
     protection): unless the mod provably computes from its index arguments alone, the part of the grid past
     the real lengths is evaluated with indices clamped to the last real position, which is what an
-    out-of-range gather yields under XLA."""
+    out-of-range gather yields under XLA.
+
+    `b_range` / `h_range` / `q_range` restrict the evaluation to a slab (batches [b0,b1), heads [h0,h1), query
+    rows [q0,q1)); the result then covers that slab only."""
+    b0, b1 = b_range or (0, B)
+    h0, h1 = h_range or (0, H)
+    q_lo, q_hi = q_range or (0, Q)
+
     def grid(where, qs, ks, clamp=False):
         q = torch.arange(qs[0], qs[1], dtype=torch.int32, device=where).reshape(1, 1, -1, 1)
         kv = torch.arange(ks[0], ks[1], dtype=torch.int32, device=where).reshape(1, 1, 1, -1)
         if clamp:
             q, kv = q.clamp(max=Qr - 1), kv.clamp(max=KVr - 1)
-        b = torch.arange(B, dtype=torch.int32, device=where).reshape(B, 1, 1, 1)
-        h = torch.arange(H, dtype=torch.int32, device=where).reshape(1, H, 1, 1)
+        b = torch.arange(b0, b1, dtype=torch.int32, device=where).reshape(-1, 1, 1, 1)
+        h = torch.arange(h0, h1, dtype=torch.int32, device=where).reshape(1, -1, 1, 1)
         return _eval_mask(fn, b, h, q, kv).to(device)
 
     Qr, KVr = (Q, KV) if real is None else (min(real[0], Q), min(real[1], KV))
+    if q_range is not None:
+        # a slab of rows: the same three regions, cut to [q_lo, q_hi)
+        clamp = not _index_arithmetic_only(fn)
+        m = torch.zeros((b1 - b0, h1 - h0, q_hi - q_lo, KV), dtype=torch.bool, device=device)
+        q_mid = min(max(Qr, q_lo), q_hi)   # rows [q_lo, q_mid) are real, [q_mid, q_hi) lie past the end
+        if q_mid > q_lo:
+            m[:, :, :q_mid - q_lo, :KVr] = grid(device, (q_lo, q_mid), (0, KVr))
+            if KVr < KV:
+                m[:, :, :q_mid - q_lo, KVr:] = grid(device, (q_lo, q_mid), (KVr, KV), clamp)
+        if q_hi > q_mid:
+            m[:, :, q_mid - q_lo:, :] = grid(device, (q_mid, q_hi), (0, KV), clamp)
+        return m
     core = grid(device, (0, Qr), (0, KVr))
     if Qr == Q and KVr == KV:
         return core
@@ -577,8 +614,8 @@ def _fit_band(m2: torch.Tensor) -> Optional[MaskMod]:
     exactly over the whole matrix, if any."""
     Q, KV = m2.shape
     dev = m2.device
-    q = torch.arange(Q, device=dev, dtype=torch.int64).reshape(Q, 1)
-    kv = torch.arange(KV, device=dev, dtype=torch.int64).reshape(1, KV)
+    q = torch.arange(Q, device=dev, dtype=torch.int32).reshape(Q, 1)
+    kv = torch.arange(KV, device=dev, dtype=torch.int32).reshape(1, KV)
     d = q - kv
     if not bool(m2.any()):
         return MaskMod(INT_MAX, INT_MAX, -1, name="all_false")
@@ -608,11 +645,18 @@ def pack_bits(mask: torch.Tensor) -> torch.Tensor:
     W = (KV + 31) // 32
     if W * 32 != KV:
         mask = torch.nn.functional.pad(mask, (0, W * 32 - KV))
-    m = mask.reshape(*lead, W, 32).to(torch.int64)
-    weights = (1 << torch.arange(32, device=mask.device, dtype=torch.int64))
-    words = (m * weights).sum(-1)
-    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words)
-    return words.to(torch.int32).contiguous()
+    # eight entries to a byte, four bytes (little-endian) to a word: no temporary wider than the mask itself
+    weights = torch.tensor([1, 2, 4, 8, 16, 32, 64, 128], dtype=torch.uint8, device=mask.device)
+    by = (mask.reshape(*lead, W * 4, 8).to(torch.uint8) * weights).sum(-1, dtype=torch.uint8)
+    return by.contiguous().view(torch.int32).reshape(*lead, W)
+
+
+def unpack_bits(words: torch.Tensor, n: int) -> torch.Tensor:
+    """int32 words [..., W] -> bool [..., n]: the inverse of pack_bits."""
+    *lead, W = words.shape
+    by = words.contiguous().view(torch.uint8).reshape(*lead, W * 4, 1)
+    shifts = torch.arange(8, dtype=torch.uint8, device=words.device)
+    return ((by >> shifts) & 1).to(torch.bool).reshape(*lead, W * 32)[..., :n]
 
 
 def block_classes(mask: torch.Tensor) -> torch.Tensor:
@@ -660,19 +704,70 @@ def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, de
 _mask_cache: dict = {}
 
 
+_SLAB_ELEMS = 1 << 24          # mask entries evaluated at a time (the callable's own temporaries scale with this)
+_FIT_ELEMS = 1 << 25           # entries of the first rows on which band parameters are fitted
+_EAGER_T_BYTES = 64 << 20      # bitmaps up to this size get their query-packed copy right away
+
+
+def _bh_extents(fn: Callable, B: int, H: int, device) -> Tuple[int, int]:
+    """Which of the batch and head extents the callable's result has at all (1 = it broadcasts): read off the shape
+    it returns for a single position."""
+    if B == 1 and H == 1:
+        return 1, 1
+    one = dense_mask_on_device(fn, B, H, 1, 1, device, real=(1, 1))
+    Bm = one.shape[0] if one.dim() == 4 else 1
+    Hm = one.shape[1] if one.dim() == 4 else 1
+    return (B if Bm > 1 else 1), (H if Hm > 1 else 1)
+
+
+def _band_equals_bitmap(band: MaskMod, words: torch.Tensor, rows: int) -> bool:
+    """The band functor reproduces every bit of the key-packed bitmap `words` [Qp, W]."""
+    Qp, W = words.shape
+    dev = words.device
+    kv = torch.arange(W * 32, dtype=torch.int32, device=dev).reshape(1, -1)
+    zero = torch.zeros((), dtype=torch.int32, device=dev)
+    for q0 in range(0, Qp, rows):
+        q = torch.arange(q0, min(q0 + rows, Qp), dtype=torch.int32, device=dev).reshape(-1, 1)
+        m = torch.broadcast_to(band(zero, zero, q, kv), (q.numel(), W * 32))
+        if not bool(torch.equal(pack_bits(m.contiguous()), words[q0:q0 + rows])):
+            return False
+    return True
+
+
 def _lower_mask_callable(fn: Callable, B: int, H: int, Q: int, KV: int, Qp: int, KVp: int, device, real) -> MaskMod:
-    m = dense_mask_on_device(fn, B, H, Qp, KVp, device, real=real or (Q, KV))
+    """Evaluate the callable over the padded index grid one (batch, head, rows) slab at a time -- the dense
+    [B,H,Q,KV] mask is never held -- and pack each slab straight into the bitmap words and the classes of its
+    32 x 32 blocks.  If every (batch, head) turns out to carry the same mask, it is fitted to the band form or kept
+    as one broadcast bitmap."""
     name = getattr(fn, "__name__", "mask_mod")
-    full_shape = torch.broadcast_shapes(m.shape, (1, 1, Qp, KVp))
-    m = torch.broadcast_to(m, full_shape)
-    bh_indep = bool((m == m[:1, :1]).all()) if (full_shape[0] > 1 or full_shape[1] > 1) else True
-    if bh_indep:
-        band = _fit_band(m[0, 0])
-        if band is not None:
+    real = real or (Q, KV)
+    Bm, Hm = _bh_extents(fn, B, H, device)
+    rows = max(128, min(Qp, (_SLAB_ELEMS // KVp) // 128 * 128))
+    W = KVp // 32
+    bits = torch.empty((Bm, Hm, Qp, W), dtype=torch.int32, device=device)
+    blk = torch.empty((Bm, Hm, Qp // 32, KVp // 32), dtype=torch.int8, device=device)
+    same = True          # every (batch, head) seen so far equals (0, 0)
+    for b in range(Bm):
+        for h in range(Hm):
+            for q0 in range(0, Qp, rows):
+                q1 = min(q0 + rows, Qp)
+                m = dense_mask_on_device(fn, B, H, Qp, KVp, device, real=real, b_range=(b, b + 1), h_range=(h, h + 1),
+                                         q_range=(q0, q1))[0, 0]
+                bits[b, h, q0:q1] = pack_bits(m)
+                blk[b, h, q0 // 32:q1 // 32] = block_classes(m)
+                if same and (b or h):
+                    same = bool(torch.equal(bits[b, h, q0:q1], bits[0, 0, q0:q1]))
+    if same:
+        # the closed band form: parameters are fitted on the first rows (_FIT_ELEMS entries) and then
+        # checked against EVERY word of the bitmap, slab by slab; a band whose window is longer than the fitted rows
+        # fails that check and stays a bitmap
+        bits, blk = bits[:1, :1].contiguous(), blk[:1, :1].contiguous()   # (lets go of the per-(batch, head) arrays)
+        fit_rows = min(Qp, max(128, (_FIT_ELEMS // KVp) // 128 * 128))
+        band = _fit_band(unpack_bits(bits[0, 0, :fit_rows], KVp))
+        if band is not None and _band_equals_bitmap(band, bits[0, 0], rows):
             band.__name__ = name
             return band
-        m = m[:1, :1]
-    # packed along the key axis for the kernels whose lanes own a query row, and along the query axis for the
-    # dK/dV kernel, whose lanes own a key
-    return MaskMod(name=name, bits=pack_bits(m.contiguous()), fn=fn, bits_t=pack_bits(m.transpose(-1, -2).contiguous()),
-                   blk=block_classes(m))
+    spec = MaskMod(name=name, bits=bits, fn=fn, blk=blk)
+    if bits.numel() * 4 <= _EAGER_T_BYTES:
+        spec.ensure_transposed()
+    return spec

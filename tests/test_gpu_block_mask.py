@@ -132,3 +132,28 @@ def test_band_closed_form_matches_brute_force(dev, seed):
         return (d >= lo) & ((d <= hi) | (kv_idx <= sink))
     bm = fa.create_block_mask(mask, 1, 2, Q, KV, BLOCK_SIZE=bs, device=dev)
     check(bm, ref_create_block_mask(omask, 1, 2, Q, KV, BLOCK_SIZE=bs))
+
+
+def test_head_and_batch_dependent_callable_at_config4_size(dev):
+    """An untagged callable that depends on the batch and the head index, at [4,16,8192,8192]: the dense mask would be
+    4.3 GB of booleans; it is evaluated in slabs and packed straight into bitmap words, so that building the block
+    mask stays below 1 GiB of device memory, and the lists are the oracle's bit for bit."""
+    import flaxattention_amd as fa
+    B, H, L = 4, 16, 8192
+
+    def mask(b, h, q_idx, kv_idx):
+        return (q_idx >= kv_idx) & (((q_idx - kv_idx) <= 256 * (h + 1) + 64 * b) | (kv_idx < 4))
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
+    base = torch.cuda.memory_allocated(dev)
+    bm = fa.create_block_mask(mask, B, H, L, L, device=dev)
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated(dev) - base
+    print(f"  peak device memory while building: {peak / 2 ** 20:.0f} MiB", flush=True)
+    assert peak < 2 ** 30
+    assert bm.spec.bits is not None and tuple(bm.spec.bits.shape) == (B, H, L, L // 32)
+    for b0, h0 in ((0, 0), (3, 15), (2, 5)):
+        ref = ref_create_block_mask(lambda b, h, q, kv: mask(b + b0, h + h0, q, kv), 1, 1, L, L)
+        for f in ("kv_num_blocks", "kv_indices", "full_kv_num_blocks", "full_kv_indices", "q_num_blocks", "q_indices",
+                  "full_q_num_blocks", "full_q_indices"):
+            assert (getattr(bm, f)[b0, h0].cpu().numpy() == ref[f][0, 0]).all(), (f, b0, h0)
