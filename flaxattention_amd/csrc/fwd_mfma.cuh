@@ -14,8 +14,9 @@
 //   S^T[kv, q]  = K_step . Q^T          D/16 v_mfma_f32_32x32x16
 //   online softmax in the accumulator layout: a lane holds 16 of the 32 scores
 //   of ONE query row, the other 16 sit in lane ^ 32 -> row max/sum are
-//   in-register reductions plus one permlane32 swap; the reference maximum only
-//   moves when it is beaten by 2^8, so the accumulator is rarely rescaled
+//   in-register reductions plus one permlane32 swap; the reference value of the
+//   exponents is not a running maximum: it moves only when a block's exponentials
+//   leave the safe range, so there is no max tree and the accumulator is rarely rescaled
 //   O^T[d, q] += V_step^T . P^T         D/16 v_mfma (P^T is already in B-operand
 //   layout; V^T fragments come from transposing LDS reads)
 #pragma once
@@ -91,10 +92,13 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
     n_full = (p.Lkv + BN - 1) / BN;
     if (!mask_hides_nothing(p.mask)) { n_part = n_full; n_full = 0; }
   }
+  // Visiting order: partial tiles first, then the fully visible ones, each from the last key tile to the first.
+  // Under causal-like masks with a score_mod that favours recent keys (ALiBi, relative-position biases) the largest
+  // scores of a row are then met first, and the row's exponent reference, once set, never has to move again.
   const int nt = n_full + n_part;
   auto tile_at = [&](int it) -> int {
-    if (!full_idx) return it;
-    return it < n_full ? full_idx[it] : part_idx[it - n_full];
+    if (!full_idx) return nt - 1 - it;
+    return it < n_part ? part_idx[n_part - 1 - it] : full_idx[n_full - 1 - (it - n_part)];
   };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
@@ -127,7 +131,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   float m_run[RQ], l_run[RQ];
 #pragma unroll
   for (int a = 0; a < RQ; a++) {
-    m_run[a] = -INFINITY;
+    m_run[a] = 0.f;  // reference value of the row's exponents; moved only by the guard in the loop
     l_run[a] = 0.f;
     if constexpr (PASS == kFwdNorm) {
       // the row's log-sum-exp from the first pass takes the place of the running reference maximum and never
@@ -141,7 +145,10 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       for (int r = 0; r < 16; r++) oacc[a][db][r] = 0.f;
   }
 
-  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  // the reference value of a row's exponents moves only when a lane's share of a block's row sum exceeds kPGuard
+  // (fp16 tops out at 65504; sums are kept in fp32) or when a row that has accumulated nothing sees a block whose
+  // exponentials are all below kPTiny
+  constexpr float kPGuard = 32768.f, kPTiny = 1.f / 64.f;
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
   // prologue: tile 0 into stage 0, tile 1 into registers
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   __syncthreads();
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
-    const bool masked = (it >= n_full) || (kv0 + BN > p.Lkv);
+    const bool masked = (it < n_part) || (kv0 + BN > p.Lkv);
     const T* Ks = Ksm[it & 1];
     const T* Vs = Vsm[PASS == kFwdLse ? 0 : (it & 1)];
     t_cur = t_nxt;
@@ -202,22 +209,20 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 #pragma unroll
         for (int a = 0; a < RQ; a++) sacc[a] = Frag<T>::mfma(kfr[s], qf[a][s], sacc[a]);
 
-      // The query blocks of the wave go through each phase together: their
-      // dependency chains (max tree, lane-half swap, exp) are independent and
-      // interleave, and one branch covers the rare rescale of either block.
-      float m_use[RQ], m_rel[RQ];
-      bool need[RQ], any_need = false;
+      // Exponents are taken relative to a per-row reference value (m_run) that is NOT a running maximum: it stays
+      // where it is until the guard below finds that a block's exponentials have left the safe range.  That saves
+      // the max tree, the lane-half exchange and a branch per block.
 #pragma unroll
       for (int a = 0; a < RQ; a++) {
         const int q_row = q_row0 + 32 * a;
-        // ---- score_mod relative to the running reference max, tile mask where needed ----
-        m_use[a] = (PASS != kFwdNorm && m_run[a] == -INFINITY) ? 0.f : m_run[a];
+        // ---- score_mod relative to the reference, tile mask where needed ----
+        const float m_use = m_run[a];
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float s0 = sacc[a][r], s1 = sacc[a][r + 1];
           if (ROUND_S) round_pair<T>(s0, s1);
-          sacc[a][r] = sm.apply_sub(s0, acc_row(r), m_use[a]);
-          sacc[a][r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use[a]);
+          sacc[a][r] = sm.apply_sub(s0, acc_row(r), m_use);
+          sacc[a][r + 1] = sm.apply_sub(s1, acc_row(r + 1), m_use);
         }
         if (cls == kBlockMixed) {
           // a real branch: every input of the mask arithmetic passes through this asm, so that
@@ -228,65 +233,66 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
           mask_block_q<BITS, BITS>(sacc[a], p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
         }
       }
-      // ---- online softmax; the reference max moves only when it is beaten by 2^kTau ----
-      if constexpr (PASS != kFwdNorm) {
-#pragma unroll
-      for (int a = 0; a < RQ; a++) m_rel[a] = block_max(sacc[a]);
 #pragma unroll
       for (int a = 0; a < RQ; a++) {
-        m_rel[a] = xhalf_max(m_rel[a]);
-        need[a] = (m_rel[a] > kTau) || (m_run[a] == -INFINITY && m_rel[a] > -INFINITY);
-        any_need |= need[a];
-      }
-      }
-      if (PASS != kFwdNorm && __any(any_need)) {
-#pragma unroll
-        for (int a = 0; a < RQ; a++) {
-          float m_opaque = m_rel[a];
-          asm volatile("" : "+v"(m_opaque));  // keeps this rare path a real branch (never if-converted)
-          const float delta = need[a] ? m_opaque : 0.f;
-          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
-          m_run[a] = need[a] ? (m_use[a] + m_rel[a]) : m_run[a];
-          l_run[a] *= alpha;
-#pragma unroll
-          for (int r = 0; r < 16; r++) sacc[a][r] -= delta;
-          if constexpr (PASS == kFwdOnePass) {
-#pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-              for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
-          }
-        }
-      }
-      if constexpr (PASS == kFwdLse) {
-        // only the row sums, in fp32 (the dense path sums the unrounded exponentials)
-#pragma unroll
-        for (int a = 0; a < RQ; a++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) l_run[a] += fast_exp2(sacc[a][r]);
-      } else {
-#pragma unroll
-      for (int a = 0; a < RQ; a++) {
+        // ---- exponentials; P rounded to the input dtype (not in the log-sum-exp pass, which sums in fp32 what
+        // the dense path sums: the unrounded exponentials); l_blk = this lane's share of the block's row sum ----
         vec8 pf[2];
+        float l_blk = 0.f;
+        auto exponentials = [&](float shift) {
+          l_blk = 0.f;
+          if constexpr (PASS == kFwdLse) {
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++) {
-          typename Pair<T>::v2 pr[4];
+            for (int r = 0; r < 16; r++) l_blk += fast_exp2(sacc[a][r] - shift);
+          } else {
 #pragma unroll
-          for (int e = 0; e < 4; e++) {
-            const float p0 = fast_exp2(sacc[a][8 * tt + 2 * e]);
-            const float p1 = fast_exp2(sacc[a][8 * tt + 2 * e + 1]);
-            pr[e] = Pair<T>::pack(p0, p1);
-            if constexpr (PASS == kFwdOnePass) l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+            for (int tt = 0; tt < 2; tt++) {
+              typename Pair<T>::v2 pr[4];
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                const float p0 = fast_exp2(sacc[a][8 * tt + 2 * e] - shift);
+                const float p1 = fast_exp2(sacc[a][8 * tt + 2 * e + 1] - shift);
+                pr[e] = Pair<T>::pack(p0, p1);
+                if constexpr (PASS == kFwdOnePass) l_blk = Pair<T>::add_sum(pr[e], l_blk);
+              }
+              pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+            }
           }
-          pf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        };
+        exponentials(0.f);
+        if constexpr (PASS != kFwdNorm) {
+          if (__any(l_blk > kPGuard || (l_run[a] == 0.f && l_blk < kPTiny))) {
+            // Rare: the exponents of this block lie far from the reference -- so far above that P nears the top of
+            // the 16-bit range, or, for a row that has accumulated nothing yet, so far below that P loses its
+            // precision (or the block is masked out for the row: then nothing moves).  Move the row's reference to
+            // the block's row maximum, rescale what the row has accumulated and redo the block's exponentials.
+            float m_rel = xhalf_max(block_max(sacc[a]));
+            asm volatile("" : "+v"(m_rel));  // keeps this rare path a real branch (never if-converted)
+            const float l_prev = xhalf_sum(l_run[a]), l_row = xhalf_sum(l_blk);  // row values: both lane halves agree
+            const bool fresh = l_prev == 0.f;                                      // nothing accumulated: nothing to rescale
+            const bool move = m_rel > -INFINITY && ((l_row > kPGuard && m_rel > 0.f) || (fresh && l_row < 2.f * kPTiny));
+            const float delta = move ? m_rel : 0.f;
+            const float alpha = fresh ? 1.f : fast_exp2(-delta);
+            m_run[a] += delta;
+            l_run[a] *= alpha;
+            if constexpr (PASS == kFwdOnePass) {
+#pragma unroll
+              for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
+            }
+            exponentials(delta);
+          }
+          l_run[a] += l_blk;
         }
-        // ---- O^T += V^T . P^T (issued before the next block's exponentials so the two overlap) ----
+        if constexpr (PASS != kFwdLse) {
+          // ---- O^T += V^T . P^T ----
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
+          for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-          for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+            for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+        }
       }
-      }  // not the log-sum-exp pass
       }  // block not entirely hidden
       if (nb == 0 && it + 1 < nt) {
         // the other stage was last read before the previous barrier: refill it with the
@@ -330,8 +336,9 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 // so that the matrix pipe and the vector ALU of a SIMD run at the same time
 // even when the waves of a workgroup march in lockstep:
 //   region A: scale / score_mod of S(u)            ||  S^T = K.Q^T of unit u+1
-//   (tile mask if needed, row max, rare rescale of the accumulator)
+//   (tile mask if needed)
 //   region B: exponentials, rounding, row sum      ||  O^T += V^T.P^T of unit u-1
+//   (guard: rare move of the row's reference value with a rescale of the accumulator)
 // Every matrix result is first read at least half a unit after it was issued.
 // Unit u-1 and unit u+1 belong to the wave's other query block, so a rescale in
 // unit u never touches an accumulator that a matrix instruction is writing.
@@ -443,7 +450,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   float m_run[RQ], l_run[RQ];
 #pragma unroll
   for (int a = 0; a < RQ; a++) {
-    m_run[a] = -INFINITY;
+    m_run[a] = 0.f;  // reference value of the row's exponents; moved only by the guard below
     l_run[a] = 0.f;
 #pragma unroll
     for (int db = 0; db < DB; db++)
@@ -459,7 +466,9 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
     for (int db = 0; db < DB; db++) vfr[tt][db] = pf[tt];
   }
 
-  constexpr float kTau = 8.f;  // lazy rescale: keep the running reference max until it is beaten by 2^8
+  // the reference value of a row's exponents stays where the row's first visible block put it until a lane's share of
+  // a block's row sum exceeds this (fp16 tops out at 65504; sums are kept in fp32)
+  constexpr float kPGuard = 32768.f, kPTiny = 1.f / 64.f;
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;   // tile it + 1
   int t_nx2 = nt > 2 ? tile_at(2) : 0;   // tile it + 2
@@ -506,13 +515,13 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
         }
         if (a == 1) read_v(Vs, nb);              // V columns of this step, first used in region B
 
-        // ---- region A: S^T of the next unit || score_mod relative to the running reference max ----
+        // ---- region A: S^T of the next unit || score_mod relative to the row's reference value ----
         float16_t s_nxt;
 #pragma unroll
         for (int r = 0; r < 16; r++) s_nxt[r] = 0.f;
 #pragma unroll
         for (int s = 0; s < DS; s++) s_nxt = Frag<T>::mfma(kfr[s], qf[1 - a][s], s_nxt);
-        const float m_use = (m_run[a] == -INFINITY) ? 0.f : m_run[a];
+        const float m_use = m_run[a];
         sm.tile(q_row, kv0 + nb * 32 + 4 * g);
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
@@ -542,28 +551,13 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
             }
           }
         }
-        // ---- row max; the reference max moves only when it is beaten by 2^kTau ----
-        float m_rel = xhalf_max(block_max(s_cur));
-        const bool need = (m_rel > kTau) || (m_run[a] == -INFINITY && m_rel > -INFINITY);
-        if (__any(need)) {
-          asm volatile("" : "+v"(m_rel));  // keeps this rare path a real branch (never if-converted)
-          const float delta = need ? m_rel : 0.f;
-          const float alpha = (m_run[a] == -INFINITY) ? 0.f : fast_exp2(-delta);
-          m_run[a] = need ? (m_use + m_rel) : m_run[a];
-          l_run[a] *= alpha;
-#pragma unroll
-          for (int r = 0; r < 16; r++) s_cur[r] -= delta;
-#pragma unroll
-          for (int db = 0; db < DB; db++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
-        }
         // ---- region B: O^T += V^T.P^T of the previous unit || exponentials, rounding, row sum ----
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
 #pragma unroll
           for (int db = 0; db < DB; db++) oacc[1 - a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[1 - a][db]);
         vec8 pn[2];
+        float l_blk = 0.f;  // this lane's share of the block's row sum
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
           typename Pair<T>::v2 pr[4];
@@ -572,7 +566,7 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
             const float p0 = fast_exp2(s_cur[8 * tt + 2 * e]);
             const float p1 = fast_exp2(s_cur[8 * tt + 2 * e + 1]);
             pr[e] = Pair<T>::pack(p0, p1);
-            l_run[a] = Pair<T>::add_sum(pr[e], l_run[a]);
+            l_blk = Pair<T>::add_sum(pr[e], l_blk);
           }
           pn[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
         }
@@ -584,6 +578,37 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
           __builtin_amdgcn_sched_group_barrier(0x400, 4, 0);             // four exponentials
           __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // rounding and row sum of the previous four
         }
+        if (__any(l_blk > kPGuard || (l_run[a] == 0.f && l_blk < kPTiny))) {
+          // Rare: the exponents of this block lie far from the reference -- so far above that P nears the top of the
+          // 16-bit range, or, for a row that has accumulated nothing yet, so far below that P loses its precision.
+          // Move the row's reference to the block's row maximum, rescale what the row has accumulated and redo the
+          // block's exponentials (s_cur still holds the exponents; the block's P has not been multiplied into V yet).
+          float m_rel = xhalf_max(block_max(s_cur));
+          asm volatile("" : "+v"(m_rel));
+          const float l_prev = xhalf_sum(l_run[a]), l_row = xhalf_sum(l_blk);   // row values: both lane halves agree
+          const bool fresh = l_prev == 0.f;                                       // nothing accumulated: nothing to rescale
+          const bool move = m_rel > -INFINITY && ((l_row > kPGuard && m_rel > 0.f) || (fresh && l_row < 2.f * kPTiny));
+          const float delta = move ? m_rel : 0.f;
+          const float alpha = fresh ? 1.f : fast_exp2(-delta);
+          m_run[a] += delta;
+          l_run[a] *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[a][db][r] *= alpha;
+          l_blk = 0.f;
+#pragma unroll
+          for (int tt = 0; tt < 2; tt++) {
+            typename Pair<T>::v2 pr[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              pr[e] = Pair<T>::pack(fast_exp2(s_cur[8 * tt + 2 * e] - delta), fast_exp2(s_cur[8 * tt + 2 * e + 1] - delta));
+              l_blk = Pair<T>::add_sum(pr[e], l_blk);
+            }
+            pn[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+          }
+        }
+        l_run[a] += l_blk;
         pf[0] = pn[0];
         pf[1] = pn[1];
         s_cur = s_nxt;
