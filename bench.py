@@ -418,7 +418,7 @@ def run_config5(dev, steps, warmup, sweep=True):
     for ql in (1, 16, 64):
         byts = 2 * 8 * 8 * Lkv * 64 * 2 + 2 * 8 * 8 * ql * 64 * 2
         best = None
-        for splits in ((8, 12, 16) if sweep else (8,)):
+        for splits in ((4, 8, 12) if sweep else (4,)):
             prs = [Prepared(dev, torch.float16, 8, 8, 8, ql, Lkv, 64, generate_alibi_bias(8, -1.0), offset_causal_mask(Lkv - ql),
                             decode_splits=splits, seed=s) for s in range(n_sets)]
             turn = [0]

@@ -24,10 +24,15 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8;
   constexpr int RPI = 64 / CPR;        // V rows one wave-wide fetch instruction fills
   constexpr int NVI = kStep / RPI;     // fetch instructions per step
-  // V strips: per wave two stages of 32 unpadded swizzled rows, filled global -> LDS directly (no staging
+  // V strips: per wave NSTG stages of 32 unpadded swizzled rows, filled global -> LDS directly (no staging
   // registers).  The same memory serves the cross-wave reduction of the partial outputs at the end.
+  // NSTG V strips per wave and DEPTH = NSTG - 1 steps of loads in flight while one is computed.  Three strips and two
+  // sets of K registers (two steps ahead) were measured at D = 64 and change nothing (config 5, one workgroup per
+  // compute unit: 53.2 us against 52.9 us at q_len 1, 57.1 against 55.7 at q_len 64): the bytes in flight are not what
+  // limits this kernel, so two strips and one step ahead it stays.
+  constexpr int NSTG = 2, DEPTH = NSTG - 1;
   constexpr int kStripElems = kStep * D;
-  constexpr int kVsBytes = 4 * 2 * kStripElems * (int)sizeof(T), kRedBytes = 4 * 16 * 64 * (int)sizeof(float);
+  constexpr int kVsBytes = 4 * NSTG * kStripElems * (int)sizeof(T), kRedBytes = 4 * 16 * 64 * (int)sizeof(float);
   __shared__ __align__(16) unsigned char vs_red[kVsBytes > kRedBytes ? kVsBytes : kRedBytes];
   __shared__ float mbuf[4][NB][32];
   // two column blocks at D = 128: the Q fragments (64 registers) are re-read from LDS every step instead
@@ -63,14 +68,29 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   }
   if (kQInLds) __syncthreads();
 
-  // schedule: list entries (64-key tiles of the query block the rows sit in) when given at that
-  // granularity, with all rows in one query block, and G == 1; else every step with the mask
-  // evaluated in each
+  // schedule, in this order of preference:
+  //  (1) a band mask whose visible keys form ONE range for the rows of this call (no sink keys, or no window): the
+  //      range follows from the mask parameters by scalar arithmetic, so the steps are walked linearly and no list is
+  //      read at all (a list lookup is a dependent global load in front of every K / V fetch: 6 us of a 59 us call);
+  //  (2) list entries (64-key tiles of the query block the rows sit in) when given at that granularity, with all
+  //      rows in one query block, and G == 1;
+  //  (3) every step, with the mask evaluated in each.
   const FlexTileLists& tl = p.tiles;
   const int32_t* full_idx = nullptr;
   const int32_t* part_idx = nullptr;
-  int n_full = 0, steps_total;
-  if (tl.kv_num && G == 1 && tl.kv_block == 2 * kStep && p.q_index_base % tl.q_block + p.Lq <= tl.q_block) {
+  int n_full = 0, steps_total, step_lo = 0;
+  const int q_lo = p.q_index_base, q_hi = p.q_index_base + p.Lq - 1;  // rows of this call
+  const bool one_range = p.mask.kind == FLEX_MASK_BAND && (p.mask.hi >= kBig || p.mask.sink < 0);
+  // keys every row sees / some row sees, from d = q + q_offset - kv, d >= lo && d <= hi
+  const int vis_hi_all = min(clamp_big(q_lo + p.mask.q_offset) - clamp_big(p.mask.lo), kBig);   // kv <= this for the first row
+  const int vis_hi_any = min(clamp_big(q_hi + p.mask.q_offset) - clamp_big(p.mask.lo), kBig);
+  const int vis_lo_all = p.mask.hi >= kBig ? 0 : max(q_hi + p.mask.q_offset - p.mask.hi, 0);    // kv >= this for the last row
+  const int vis_lo_any = p.mask.hi >= kBig ? 0 : max(q_lo + p.mask.q_offset - p.mask.hi, 0);
+  if (one_range) {
+    const int kv_last = min(vis_hi_any, p.Lkv - 1);
+    step_lo = vis_lo_any / kStep;
+    steps_total = kv_last >= vis_lo_any ? kv_last / kStep - step_lo + 1 : 0;
+  } else if (tl.kv_num && G == 1 && tl.kv_block == 2 * kStep && p.q_index_base % tl.q_block + p.Lq <= tl.q_block) {
     const int64_t row = (b * tl.stride_b + hk * tl.stride_h) * tl.n_q_blocks + p.q_index_base / tl.q_block;
     n_full = tl.full_kv_num[row];
     const int n_part = tl.kv_num[row];
@@ -81,7 +101,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     steps_total = (p.Lkv + kStep - 1) / kStep;
   }
   auto step_kv0 = [&](int st) -> int {
-    if (!full_idx) return st * kStep;
+    if (!full_idx) return (step_lo + st) * kStep;
     const int item = st >> 1;
     const int tile = item < n_full ? full_idx[item] : part_idx[item - n_full];
     return tile * (2 * kStep) + (st & 1) * kStep;
@@ -98,12 +118,12 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   // masked out and their P is 0, so what they hold does not matter as long as
   // it is finite.
   const int last = p.Lkv - 1;
-  vec8 kfr[DS];
-  T* Vw = reinterpret_cast<T*>(vs_red) + w * 2 * kStripElems;
+  vec8 kfA[DS], kfB[DS];  // two sets of K registers, named so that they stay in registers (kfB unused at DEPTH 1)
+  T* Vw = reinterpret_cast<T*>(vs_red) + w * NSTG * kStripElems;
   const int fill_row = lane / CPR, fill_pos = lane % CPR;
   // V first, K last: loads return in order, so once the K registers of a step have arrived (the
   // compiler waits for them before the first MFMA) the V strip of that step has landed too
-  auto load_step = [&](int kv0, int stage) {
+  auto load_step = [&](vec8 (&kfr)[DS], int kv0, int stage) {
     const int lim = last - kv0;  // last valid row of this step, relative
     const T* vp = vbase + (int64_t)kv0 * vs2;
     if constexpr (PASS != kDecLse) {
@@ -153,16 +173,19 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   const bool trivial_mask = p.mask.kind == FLEX_MASK_BAND && p.mask.lo == INT32_MIN && p.mask.hi == INT32_MAX;
   constexpr float kTau = 8.f;
 
-  // KV offsets are looked up two visits ahead so that the (dependent) tile-index
-  // load never sits between a wave and its next K/V loads
+  // KV offsets are looked up four visits ahead so that the (dependent) tile-index load never sits between a wave
+  // and its next K/V loads
   int st = st_begin + w;
-  int kv_cur = st < st_end ? step_kv0(st) : 0;
-  int kv_nx1 = st + 4 < st_end ? step_kv0(st + 4) : 0;
-  int kv_nx2 = st + 8 < st_end ? step_kv0(st + 8) : 0;
+  int kv_q0 = st < st_end ? step_kv0(st) : 0;
+  int kv_q1 = st + 4 < st_end ? step_kv0(st + 4) : 0;
+  int kv_q2 = st + 8 < st_end ? step_kv0(st + 8) : 0;
+  int kv_q3 = st + 12 < st_end ? step_kv0(st + 12) : 0;
   int stage = 0;
-  if (st < st_end) load_step(kv_cur, 0);
-  for (; st < st_end; st += 4, stage ^= 1) {
-    const int kv0 = kv_cur;
+  if (st < st_end) load_step(kfA, kv_q0, 0);
+  if (DEPTH == 2 && st + 4 < st_end) load_step(kfB, kv_q1, 1);
+  // one step of this wave; kfr holds its K rows and is refilled for the step DEPTH visits later
+  auto visit = [&](vec8 (&kfr)[DS]) {
+    const int kv0 = kv_q0;
     // scores first: they consume the K registers, which the next step's loads then reuse
     float16_t s_a, s_b;  // named (not an array) so that they stay in registers
 #pragma unroll
@@ -178,14 +201,18 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
         s_b = Frag<T>::mfma(kfr[s], *reinterpret_cast<const vec8*>(qp + 32 * ROWE), s_b);
       }
     }
-    // this step's V strip landed with its K registers; the other strip was last read a step ago
-    if (st + 4 < st_end) load_step(kv_nx1, stage ^ 1);
-    kv_cur = kv_nx1;
-    kv_nx1 = kv_nx2;
-    if (st + 12 < st_end) kv_nx2 = step_kv0(st + 12);
-    // steps that come from the list of fully visible tiles need no mask evaluation
+    // this step's V strip landed with its K registers (loads return in order); the strip refilled now was last
+    // read a step ago
+    if (st + 4 * DEPTH < st_end) load_step(kfr, DEPTH == 2 ? kv_q2 : kv_q1, stage + DEPTH >= NSTG ? stage + DEPTH - NSTG : stage + DEPTH);
+    kv_q0 = kv_q1;
+    kv_q1 = kv_q2;
+    kv_q2 = kv_q3;
+    if (st + 16 < st_end) kv_q3 = step_kv0(st + 16);
+    // steps that every row of the call sees completely need no mask evaluation: those from the list of fully
+    // visible tiles, and under a one-range band mask those inside the range common to all rows
     const bool listed_full = full_idx && (st >> 1) < n_full;
-    const bool need_mask = (!trivial_mask && !listed_full) || (kv0 + kStep > p.Lkv);
+    const bool band_full = one_range && kv0 >= vis_lo_all && kv0 + kStep - 1 <= vis_hi_all;
+    const bool need_mask = (!trivial_mask && !listed_full && !band_full) || (kv0 + kStep > p.Lkv);
 
     vec8 pf[NB][2];
 #pragma unroll
@@ -261,6 +288,12 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
       }
       __builtin_amdgcn_wave_barrier();
     }
+    st += 4;
+    stage = stage + 1 == NSTG ? 0 : stage + 1;
+  };
+  while (st < st_end) {
+    visit(kfA);
+    if (DEPTH == 2 && st < st_end) visit(kfB);
   }
 
   // ---- merge the four waves ----
@@ -342,6 +375,16 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(FlexAttnParams p, c
     ms = ml.x;
     ls = ml.y;
   }
+  // the first eight splits' partial outputs are requested together with the (m, l) pairs, before anything waits:
+  // the kernel is a chain of memory latencies (its data was written by other XCDs and comes from HBM), and this
+  // way there is one of them instead of two
+  float v0[8][D / 64];
+  if (o) {
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+#pragma unroll
+      for (int a = 0; a < D / 64; a++) v0[u][a] = (u < splits) ? o_part[(u * rows + row) * D + lane + 64 * a] : 0.f;
+  }
   float m = ms;
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
   const float sc = (ms == -INFINITY) ? 0.f : fast_exp2(ms - m);
@@ -352,7 +395,13 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(FlexAttnParams p, c
   float acc[D / 64];
 #pragma unroll
   for (int a = 0; a < D / 64; a++) acc[a] = 0.f;
-  for (int s0 = 0; s0 < splits; s0 += 8) {
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const float w = __shfl(sc, u, 64);
+#pragma unroll
+    for (int a = 0; a < D / 64; a++) acc[a] = fmaf(w, v0[u][a], acc[a]);
+  }
+  for (int s0 = 8; s0 < splits; s0 += 8) {
     float v[8][D / 64];
 #pragma unroll
     for (int u = 0; u < 8; u++)

@@ -40,13 +40,12 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 }
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
-  // aim for one resident generation of workgroups on 256 CUs, as many per CU as the kernel's
-  // registers allow: D = 64: three with up to 32 query columns, two with 64; D = 128: two and one;
-  // at least 8 steps each
+  // ONE workgroup per compute unit: a bandwidth-bound kernel gains nothing from more, and every further split adds
+  // partials to write and merge (config 5 at q_len 1: 53 us with 4 splits = 256 workgroups, 54 us with 8, 58 us with
+  // 16; at q_len 64: 56 us with 4, 60 us with 8).  At least 8 steps each.
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
-  const bool wide = (p.Hq / p.Hkv) * p.Lq > 32;
-  const int slots = p.D == 64 ? (wide ? 512 : 768) : (wide ? 256 : 512);
+  const int slots = 256;
   int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;
