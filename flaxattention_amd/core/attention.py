@@ -47,8 +47,8 @@ import torch
 
 from .. import _lib
 from .blockmask import BlockMask, _create_empty_block_mask
-from .common import (IDENTITY, MaskMod, ScoreMod, _identity, _mask_mod_signature, _score_mod_signature,
-                     resolve_mask_mod, resolve_score_mod)
+from .common import (IDENTITY, MaskMod, ScoreMod, ScoreModNotLowered, _identity, _mask_mod_signature,
+                     _score_mod_signature, resolve_mask_mod, resolve_score_mod)
 
 Array = torch.Tensor
 
@@ -302,6 +302,102 @@ class _FlexAttention(torch.autograd.Function):
         return dq, dk, dv, None
 
 
+# ---- score_mods that cannot be lowered to a functor: linearised at the scores of the call ----------------------
+_LINEARISE_BYTES = 2 << 30   # dense fp32 temporaries of one batch chunk (scores, mod, derivative, the two tables)
+
+
+def _linearised_tables(score_fn, q, k, scale: float, b0: int):
+    """For an arbitrary differentiable scalar score_mod f: the scaled scores S0 of the call (the product computed in
+    the input dtype and cast to fp32, then scaled: attention.py:27, 55), Y = f(S0, b, h, q_idx, kv_idx) and
+    G = dY/dS0, as the dense fp32 tables of the affine functor  mul * s + add  with mul = G and add = Y - G * S0.
+    At s = S0 that is f(S0) exactly, its derivative is f'(S0), and where a kernel's own score differs from S0 in the
+    last bit of the input dtype the difference enters to first order.  `b0` is the batch index of q[0]."""
+    B, Hq, Lq, _ = q.shape
+    G_ = Hq // k.shape[1]
+    kk = k if G_ == 1 else k.repeat_interleave(G_, dim=1)   # the reference repeats K for GQA (attention.py:80-82)
+    s0 = (torch.matmul(q, kk.transpose(-1, -2)).to(torch.float32) * scale).requires_grad_(True)
+    dev = q.device
+    b = torch.arange(b0, b0 + B, dtype=torch.int32, device=dev).reshape(B, 1, 1, 1)
+    h = torch.arange(Hq, dtype=torch.int32, device=dev).reshape(1, Hq, 1, 1)
+    qi = torch.arange(Lq, dtype=torch.int32, device=dev).reshape(1, 1, Lq, 1)
+    ki = torch.arange(k.shape[2], dtype=torch.int32, device=dev).reshape(1, 1, 1, -1)
+    with torch.enable_grad():
+        y = torch.as_tensor(score_fn(s0, b, h, qi, ki)).to(torch.float32)
+        y = torch.broadcast_to(y, s0.shape)
+        (g,) = torch.autograd.grad(y.sum(), s0, allow_unused=True)
+    if g is None:
+        g = torch.zeros_like(s0)
+    y, s0 = y.detach(), s0.detach()
+    g = torch.where(torch.isfinite(g), g, torch.zeros_like(g))
+    add = torch.where(torch.isfinite(y), y - g * s0, y)   # (a mod that returns -inf masks the entry: keep it)
+    return g.contiguous(), add.contiguous()
+
+
+class _FlexAttentionLinearised(torch.autograd.Function):
+    """flax_attention for a score_mod outside the functor families and not affine in the score (the reference applies
+    any scalar callable, attention.py:59-63).  Per chunk of batch elements the callable and its derivative are
+    evaluated at the call's own scores and handed to the kernels as the tables of an affine functor; the backward
+    evaluates them again instead of keeping them."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, cfg):
+        score_fn, block_mask, mask_mod, scale, opts = cfg
+        B, Hq, Lq, _ = q.shape
+        per_b = 5 * Hq * Lq * k.shape[2] * 4
+        step = max(1, min(B, _LINEARISE_BYTES // max(per_b, 1)))
+        o = torch.empty((B, Hq, Lq, v.shape[3]), dtype=q.dtype, device=q.device)
+        lse2 = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
+        chunks = []
+        for b0 in range(0, B, step):
+            b1 = min(b0 + step, B)
+            plan = _FlexAttentionLinearised._chunk_plan(cfg, q[b0:b1], k[b0:b1], v[b0:b1], b0)
+            oc, lc = _run_fwd(plan, q[b0:b1], k[b0:b1], v[b0:b1])
+            o[b0:b1], lse2[b0:b1] = oc, lc
+            plan.score = None   # the tables are not kept for the backward
+            chunks.append((b0, b1))
+        ctx.save_for_backward(q, k, v, o, lse2)
+        ctx.cfg, ctx.chunks = cfg, chunks
+        ctx.set_materialize_grads(False)
+        return o, lse2
+
+    @staticmethod
+    def _chunk_plan(cfg, qc, kc, vc, b0):
+        score_fn, block_mask, mask_mod, scale, opts = cfg
+        mul, add = _linearised_tables(score_fn, qc, kc, scale, b0)
+        score = ScoreMod(_lib.SCORE_AFFINE, name=getattr(score_fn, "__name__", "score_mod"), mul=mul, add=add, fn=score_fn)
+        # the mask of this chunk: a functor that does not look at the batch index serves as it is; anything else is the
+        # user's callable with the chunk's batch offset (lowered again for the chunk)
+        src = block_mask.mask_mod if block_mask is not None else mask_mod
+        spec = block_mask.spec if block_mask is not None else (src if isinstance(src, MaskMod) else None)
+        if not (isinstance(spec, MaskMod) and (spec.bits is None or spec.bits.shape[0] == 1)):
+            spec = None if src is None else (lambda b, h, q_idx, kv_idx: src(b + b0, h, q_idx, kv_idx))
+        plan = _make_plan(qc, kc, vc, IDENTITY, None, spec, scale, opts)
+        plan.score = score
+        plan.keep = [plan.mask.bits, mul, add]
+        return plan
+
+    @staticmethod
+    def backward(ctx, d_o, d_lse2):
+        q, k, v, o, lse2 = ctx.saved_tensors
+        if d_o is None:
+            d_o = torch.zeros_like(o)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        for b0, b1 in ctx.chunks:
+            plan = _FlexAttentionLinearised._chunk_plan(ctx.cfg, q[b0:b1], k[b0:b1], v[b0:b1], b0)
+            dl = None if d_lse2 is None else d_lse2[b0:b1]
+            dq[b0:b1], dk[b0:b1], dv[b0:b1] = _run_bwd(plan, q[b0:b1], k[b0:b1], v[b0:b1], o[b0:b1], lse2[b0:b1],
+                                                        d_o[b0:b1], dl)
+        return dq, dk, dv, None
+
+
+def _attend_linearised(q, k, v, score_fn, block_mask, mask_mod, scale, kernel_options) -> Tuple[Array, Array]:
+    opts = dict(kernel_options or {})
+    opts["decode"] = False   # the split-KV decode kernel takes closed-form functors only
+    opts.pop("decode_splits", None)
+    cfg = (score_fn, block_mask, mask_mod, float(scale), opts)
+    return _FlexAttentionLinearised.apply(q, k, v, cfg)
+
+
 def _attend(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad):
         return _FlexAttention.apply(q, k, v, plan)
@@ -375,7 +471,10 @@ def math_attention(query: Array, key: Array, value: Array, score_mod: Callable, 
     q, k, v = map(_as_kernel_layout, (query, key, value))
     opts = dict(kernel_options or {})
     opts.setdefault("strict", True)
-    plan = _make_plan(q, k, v, score_mod, None, mask_mod, scale, opts)
+    try:
+        plan = _make_plan(q, k, v, score_mod, None, mask_mod, scale, opts)
+    except ScoreModNotLowered:
+        return _attend_linearised(q, k, v, score_mod, None, mask_mod, scale, opts)
     return _attend(plan, q, k, v)
 
 
@@ -413,8 +512,11 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
     if scale is None:
         scale = 1.0 / math.sqrt(query.shape[-1])
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
-    plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
-    out, lse2 = _attend(plan, q, k, v)
+    try:
+        plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
+        out, lse2 = _attend(plan, q, k, v)
+    except ScoreModNotLowered:
+        out, lse2 = _attend_linearised(q, k, v, score_mod, block_mask, None, scale, kernel_options)
     out = out[..., :value.shape[-1]]
     if return_lse:
         return out, lse2 * math.log(2.0)
@@ -465,7 +567,10 @@ def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Opt
         out, _ = _NothingToAttend.apply(query, key, value)
         return out if bhln else out.transpose(1, 2)
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
-    plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
-    out, _ = _attend(plan, q, k, v)
+    try:
+        plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
+        out, _ = _attend(plan, q, k, v)
+    except ScoreModNotLowered:
+        out, _ = _attend_linearised(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
     out = out[..., :value.shape[-1]]
     return out if bhln else out.transpose(1, 2)

@@ -285,6 +285,10 @@ def affine_score_mod(fn: Callable, B: int, H: int, Lq: int, Lkv: int, device) ->
 _score_cache: dict = {}
 
 
+class ScoreModNotLowered(NotImplementedError):
+    """resolve_score_mod: the callable is not one of the functor families and not affine in the score."""
+
+
 def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int, int, int, int]] = None,
                       device=None) -> ScoreMod:
     """Lower a score_mod callable to a kernel functor, or raise.  `shape` = (B, H, Lq, Lkv) and `device`
@@ -322,10 +326,10 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
             if stamp is not None:
                 _score_cache[key] = (fn, spec, stamp)
             return spec
-    raise NotImplementedError(
+    raise ScoreModNotLowered(
         "score_mod is neither one of the fused functor families (identity, checkerboard, ALiBi, tanh soft-cap, "
-        "relative-position bias) nor affine in the score (mul[b,h,q,kv] * score + add[b,h,q,kv]); "
-        "only those can be lowered to the kernels")
+        "relative-position bias) nor affine in the score (mul[b,h,q,kv] * score + add[b,h,q,kv]): it cannot be lowered "
+        "to a functor that is independent of the scores (the front-ends then linearise it at the scores of each call)")
 
 
 # ---------------------------------------------------------------------------

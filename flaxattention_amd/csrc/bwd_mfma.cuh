@@ -748,7 +748,8 @@ static int launch_kind(const FlexAttnParams& p, const BwdArgs& a) {
     case FLEX_SCORE_ALIBI: return launch_rs<T, D, FLEX_SCORE_ALIBI>(p, a);
     case FLEX_SCORE_TANH_SOFTCAP: return launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, a);
     case FLEX_SCORE_REL_BIAS: return launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, a);
-    case FLEX_SCORE_AFFINE: return launch_rs<T, D, FLEX_SCORE_AFFINE>(p, a);
+    case FLEX_SCORE_AFFINE:
+      return p.score.mul ? launch_rs<T, D, kScoreAffineMul>(p, a) : launch_rs<T, D, FLEX_SCORE_AFFINE>(p, a);
   }
   return 1;
 }

@@ -685,7 +685,7 @@ static void launch_rs(const FlexAttnParams& p, const FwdArgs& a) {
   // kernel with 256-row workgroups.  Otherwise the 128-row kernel: twice the workgroups, half the length of the
   // longest one, which is what bounds a causal-like schedule.
   // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
-  if constexpr (KIND != FLEX_SCORE_AFFINE && D == 64) {
+  if constexpr (KIND != FLEX_SCORE_AFFINE && KIND != kScoreAffineMul && D == 64) {
     if (!p.tiles.kv_num && mask_hides_nothing(p.mask)) {
       const bool tail = p.Lkv % kFwdBN != 0, rs = (p.flags & FLEX_ROUND_S) != 0;
       if (rs && !tail) launch_pipe_kernel<T, KIND, true, false>(p, a);
@@ -712,7 +712,10 @@ static int launch_kind(const FlexAttnParams& p, const FwdArgs& a) {
     case FLEX_SCORE_ALIBI: launch_rs<T, D, FLEX_SCORE_ALIBI>(p, a); return 0;
     case FLEX_SCORE_TANH_SOFTCAP: launch_rs<T, D, FLEX_SCORE_TANH_SOFTCAP>(p, a); return 0;
     case FLEX_SCORE_REL_BIAS: launch_rs<T, D, FLEX_SCORE_REL_BIAS>(p, a); return 0;
-    case FLEX_SCORE_AFFINE: launch_rs<T, D, FLEX_SCORE_AFFINE>(p, a); return 0;
+    case FLEX_SCORE_AFFINE:
+      if (p.score.mul) launch_rs<T, D, kScoreAffineMul>(p, a);
+      else launch_rs<T, D, FLEX_SCORE_AFFINE>(p, a);
+      return 0;
   }
   return 1;
 }

@@ -14,8 +14,8 @@ static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0
 // dtype / head size / layout the MFMA kernels can take at all
 bool flex_mfma_shape_ok(const FlexAttnParams& p) {
   if (p.dtype != FLEX_F16 && p.dtype != FLEX_BF16) return false;
-  // dense tables: an additive one is fused (read per block); a multiplicative one goes to the generic kernels
-  if (p.score.kind == FLEX_SCORE_AFFINE && (p.score.mul || !p.score.add)) return false;
+  // dense tables (additive, multiplicative or both) are read per block by the fused kernels
+  if (p.score.kind == FLEX_SCORE_AFFINE && !p.score.mul && !p.score.add) return false;
   if (p.D != p.Dv || (p.D != 64 && p.D != 128)) return false;
   if (!strides_ok(p.q_stride) || !strides_ok(p.k_stride) || !strides_ok(p.v_stride) || !strides_ok(p.o_stride)) return false;
   if ((int64_t)((p.Lq + 127) / 128) * p.Hq * p.B > 0x7fffffff) return false;

@@ -232,6 +232,54 @@ template <> struct Score2<FLEX_SCORE_AFFINE> {
   __device__ __forceinline__ float grad(float s, int off) const { return 1.f; }
 };
 
+// mul[b,h,q,kv] * score + add[b,h,q,kv] from dense fp32 tables (FLEX_SCORE_AFFINE with a multiplicative table: what
+// a score_mod that scales the score by a captured or position-dependent factor is lowered to, and what an arbitrary
+// differentiable score_mod becomes once it is linearised at the scores of the call).  Both tables' entries of a lane's
+// block are fetched when the block is entered; the derivative is the multiplicative entry itself.
+constexpr int kScoreAffineMul = 102;
+template <> struct Score2<kScoreAffineMul> {
+  static constexpr bool kGradOne = false;
+  float c;
+  const float* add_bh;
+  const float* mul_bh;
+  int64_t sq;
+  int q_last, kv_last;
+  float bias[16], fac[16];  // log2(e) * add and mul for accumulator register r
+  static __device__ __forceinline__ constexpr int reg_of(int off) { return 4 * (off / 8) + (off % 4); }
+  __device__ __forceinline__ void init(const FlexScoreMod& m, float scale, int h, int b = 0, int Lq = 0, int Lkv = 0) {
+    c = scale * kLog2e;
+    const int64_t off = b * m.stride_b + h * m.stride_h;
+    add_bh = m.add ? m.add + off : nullptr;
+    mul_bh = m.mul + off;
+    sq = m.stride_q;
+    q_last = Lq - 1;
+    kv_last = Lkv - 1;
+  }
+  __device__ __forceinline__ void tile(int q, int kvb) {
+    const int64_t row = (int64_t)min(q, q_last) * sq;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int64_t at = row + min(kvb + acc_row(r), kv_last);
+      fac[r] = mul_bh[at];
+      bias[r] = add_bh ? add_bh[at] * kLog2e : 0.f;
+    }
+  }
+  __device__ __forceinline__ void tileT(int qb, int kv) {
+    const int col = min(kv, kv_last);
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int64_t at = (int64_t)min(qb + acc_row(r), q_last) * sq + col;
+      fac[r] = mul_bh[at];
+      bias[r] = add_bh ? add_bh[at] * kLog2e : 0.f;
+    }
+  }
+  __device__ __forceinline__ float apply(float s, int off) const { return fmaf(s * fac[reg_of(off)], c, bias[reg_of(off)]); }
+  __device__ __forceinline__ float apply_sub(float s, int off, float m) const {
+    return fmaf(s * fac[reg_of(off)], c, bias[reg_of(off)] - m);
+  }
+  __device__ __forceinline__ float grad(float s, int off) const { return fac[reg_of(off)]; }
+};
+
 // band / bitmap mask evaluated at (q, kv)
 struct Mask2 {
   MaskEval ev;

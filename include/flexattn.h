@@ -39,9 +39,10 @@ enum FlexScoreKind {
   FLEX_SCORE_AFFINE = 5        /* mul[b,h,q,kv] * score + add[b,h,q,kv] from dense fp32
                                   tables: what a Python score_mod that is affine in the score
                                   (captured bias tables, position-dependent scaling;
-                                  attention.py:22-23, 59-63) is lowered to.  An additive
-                                  table alone (mul == NULL) is read by the fused kernels;
-                                  with a multiplicative table the generic kernels serve it. */
+                                  attention.py:22-23, 59-63) is lowered to, and what an arbitrary
+                                  differentiable score_mod becomes when it is linearised at the
+                                  scores of the call.  The fused kernels read both tables
+                                  (16 entries per lane and 32x32 block).  */
 };
 
 typedef struct FlexScoreMod {

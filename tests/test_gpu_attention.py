@@ -248,9 +248,10 @@ def test_untagged_score_mod_is_recognised(dev):
 
     def unknown(score, b, h, q_idx, kv_idx):
         return score * score
-    q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 32, torch.float32))
-    with pytest.raises(NotImplementedError):
-        fa.flax_attention(q, k, v, score_mod=unknown)
+    # outside every family and not affine in the score: served by linearisation at the call's scores
+    q, k, v = seeded_qkv(1, 2, 2, 16, 16, 32, torch.float32)
+    out = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=unknown)
+    assert rel_l2(out.cpu(), ref_attention(q, k, v, unknown, None)) <= 1e-4
 
 
 def test_errors(dev):
@@ -340,6 +341,34 @@ def test_fused_forward_exponent_reference_guard(dev, dtype):
         assert float(want_lse.max()) < -100.0   # the case is what it claims to be
         close(out, want, dtype, f"O, scores far below zero, mask {mask is not None}", fast_bf16)
         assert torch.isfinite(lse).all() and max_abs(lse.cpu(), want_lse) <= 2e-2 * max(1.0, want_lse.abs().max().item() / 64)
+
+
+ARBITRARY = [
+    ("square", lambda s, b, h, q, kv: 0.1 * s * s + s),
+    ("sin", lambda s, b, h, q, kv: 3.0 * torch.sin(s) + 0.01 * (kv - q)),
+    ("leaky_by_head", lambda s, b, h, q, kv: torch.where(s > 0, s, 0.25 * (h + 1) * s)),
+    ("batch_dependent", lambda s, b, h, q, kv: s * torch.sigmoid(s) * (1.0 + 0.5 * b)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32], ids=["f16", "bf16", "f32"])
+@pytest.mark.parametrize("name,fn", ARBITRARY, ids=[a[0] for a in ARBITRARY])
+def test_arbitrary_score_mod_is_linearised(dev, dtype, name, fn):
+    """A score_mod that is neither one of the functor families nor affine in the score (the reference applies any
+    scalar callable, attention.py:59-63): evaluated, with its derivative, at the scores of the call and handed to the
+    kernels as dense tables.  Forward, lse and all three gradients against the oracle, which applies the same callable
+    densely and differentiates it with autograd; batch of 3 in chunks, GQA, ragged lengths, causal mask."""
+    import flaxattention_amd.core.attention as att
+    print(f"case arbitrary score_mod {name} {dtype}", flush=True)
+    old = att._LINEARISE_BYTES
+    att._LINEARISE_BYTES = 5 * 4 * 200 * 333 * 4 * 2   # two batch elements per chunk: the batch of 3 takes two chunks
+    try:
+        run(dev, dtype, 3, 4, 2, 200, 333, 64, score=fn, oscore=fn, mask=causal_mask, omask=o_causal_mask,
+            strict=False, scale_maxabs=True)
+        run(dev, dtype, 3, 2, 2, 130, 130, 128 if dtype != torch.float32 else 32, score=fn, oscore=fn, strict=False,
+            pallas=True, scale_maxabs=True)
+    finally:
+        att._LINEARISE_BYTES = old
 
 
 def test_lse_is_differentiable(dev):
@@ -555,9 +584,13 @@ def test_affine_score_mod_tables(dev):
 
     def quadratic(score, b, h, q_idx, kv_idx):
         return score * score
-    q, k, v = (t.to(dev) for t in seeded_qkv(1, 2, 2, 16, 16, 64, torch.float16))
-    with pytest.raises(NotImplementedError):
-        fa.flax_attention(q, k, v, score_mod=quadratic)
+    # not affine in the score: no score-independent functor exists, the front-end linearises it per call
+    from flaxattention_amd.core.common import ScoreModNotLowered, resolve_score_mod
+    with pytest.raises(ScoreModNotLowered):
+        resolve_score_mod(quadratic, 2, (1, 2, 16, 16), dev)
+    q, k, v = seeded_qkv(1, 2, 2, 16, 16, 64, torch.float16)
+    out = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=quadratic)
+    assert rel_l2(out.cpu(), ref_attention(q, k, v, quadratic, None)) <= 1e-3
 
 
 @pytest.mark.parametrize("shape", [(2, 2, 0, 64, 64), (2, 2, 16, 0, 64), (0, 2, 16, 64, 64), (1, 2, 300, 0, 128)])
