@@ -10,8 +10,8 @@ out.sum()); one step = forward kernel + both backward kernels.  The last line
 printed on stdout is ONE JSON object (the driver's contract).  Besides the
 headline it carries the decode half of the metric (configuration 5, q_len 1,
 16 and 64 over rotating KV caches: us, GB/s, fraction of 8 TB/s), the step
-times of configurations 3 and 4, and every training configuration in both
-numerics modes ("fast" and "parity"); --all adds the probes, the split sweep
+times of configurations 3 and 4, and every training configuration in the three
+numerics modes ("fast", "parity", "unrounded"); --all adds the probes, the split sweep
 of the decode kernel and the block-mask builder.
 
 Kernel durations are HIP-event intervals taken INSIDE the step (forward, dQ
@@ -246,7 +246,7 @@ def run_train_config(dev, name, steps, warmup, opts=None, graph=False):
     else:
         ms = wall_time_ms(step, steps, warmup)
     n = max(steps, 10)
-    parity = bool(pr.p.flags & pr._lib.FLAG_PARITY)
+    parity = bool(pr.p.flags & (pr._lib.FLAG_PARITY | pr._lib.FLAG_UNROUNDED))   # two launches in the dQ call
     # D = 64: the pipelined kernel runs when there are no tile lists and the numerics are "fast", the list-driven
     # kernel otherwise (twice in the parity numerics: log-sum-exp pass, then the normalised pass)
     fwd_name = "fwd_pipe_kernel" if (pr.block_mask is None and not parity) else "fwd_mfma_kernel"
@@ -453,7 +453,7 @@ def main():
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (no other configurations, modes or decode)")
     ap.add_argument("--all", action="store_true", help="also the probes, the decode split sweep and the block-mask builder (in 'extra')")
     ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
-    ap.add_argument("--numerics", default=None, choices=["fast", "parity"],
+    ap.add_argument("--numerics", default=None, choices=["fast", "parity", "unrounded"],
                     help="numerics of the headline workload (default: the library's: fp16 fast, bf16 parity)")
     ap.add_argument("--graph", action="store_true", help="replay the three kernels of a step as one HIP graph instead of launching them eagerly")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -493,7 +493,7 @@ def main():
                                    "prefill_kernel_us": round(d["prefill_kernel_us"], 1)} for ql, d in c5.items()}}
         # every training configuration in both numerics modes
         c4 = {}
-        for num in ("parity", "fast"):
+        for num in ("unrounded", "parity", "fast"):
             x = run_config4(dev, a.steps, a.warmup, dict(opts, numerics=num))
             c4[num] = {"fwd_us": round(x["us"], 1), "fwd_tflops": round(x["tflops"], 1),
                        "pct_mfma_peak": round(x["tflops"] / PEAK_MFMA_TFLOPS * 100, 2), "default": num == "parity"}
@@ -501,7 +501,7 @@ def main():
         modes = {}
         for wl, default in (("config3", "parity"), ("config2", "fast")):
             modes[wl] = {}
-            for num in ("parity", "fast"):
+            for num in ("unrounded", "parity", "fast"):
                 rr = run_train_config(dev, wl, a.steps, a.warmup, dict(opts, numerics=num))
                 modes[wl][num] = mode_summary(rr)
                 modes[wl][num]["default"] = num == default

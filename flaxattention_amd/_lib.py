@@ -18,6 +18,7 @@ FLEX_F32, FLEX_F16, FLEX_BF16 = 0, 1, 2
 SCORE_IDENTITY, SCORE_CHECKERBOARD, SCORE_ALIBI, SCORE_TANH_SOFTCAP, SCORE_REL_BIAS, SCORE_AFFINE = range(6)
 MASK_BAND, MASK_BITS = 0, 1
 FLAG_ROUND_S, FLAG_STRICT, FLAG_FORCE_GENERIC, FLAG_BWD_ONLY_DQ, FLAG_BWD_ONLY_DKV, FLAG_PARITY = 1, 2, 4, 8, 16, 32
+FLAG_UNROUNDED = 64
 INT_MIN, INT_MAX = -(2 ** 31), 2 ** 31 - 1
 
 

@@ -21,6 +21,14 @@ selects numerics here:
                         faster.  Default: "parity" for bfloat16, whose 8-bit
                         mantissa puts "fast" 3e-3 (relative L2) away from the dense
                         path, and "fast" for float16, where it stays within 1e-3.
+                        "unrounded": no internal round trip at all -- S is not
+                        rounded, P and dS enter the matrix products as a high and
+                        a low part (twice the mantissa), delta = sum_j P dP from an
+                        unrounded row sweep; only the results are rounded.  What
+                        the dense path computes if XLA removes the round trips of
+                        attention.py:27, 104-105 (excess-precision simplification);
+                        within 1e-4 of that variant of the oracle, about 1.6x the
+                        time of "fast".
     {"strict": True}    faithful kernels on the vector ALU: the same rounding
                         points as "parity", any dtype and head size
     {"round_s": bool}   fused kernels: round Q.K^T through the input dtype
@@ -160,10 +168,12 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
     if opts.get("backend", "auto") == "generic":
         flags |= _lib.FLAG_FORCE_GENERIC
     numerics = opts.get("numerics", "parity" if q.dtype == torch.bfloat16 else "fast")
-    if numerics not in ("parity", "fast"):
-        raise ValueError(f'kernel_options["numerics"] must be "parity" or "fast", got {numerics!r}')
+    if numerics not in ("parity", "fast", "unrounded"):
+        raise ValueError(f'kernel_options["numerics"] must be "parity", "fast" or "unrounded", got {numerics!r}')
     if numerics == "parity" and q.dtype != torch.float32:
         flags |= _lib.FLAG_PARITY
+    if numerics == "unrounded":
+        flags = (flags & ~(_lib.FLAG_ROUND_S | _lib.FLAG_STRICT)) | _lib.FLAG_UNROUNDED
     plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, score, flags, opts))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and opts.get("tile_lists", True) and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
@@ -192,7 +202,8 @@ def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
     B, Hq, Lq, D = q.shape
     G = Hq // k.shape[1]
     ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
-          and score.kind != _lib.SCORE_AFFINE and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)))
+          and score.kind != _lib.SCORE_AFFINE
+          and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC | _lib.FLAG_UNROUNDED)))
     if want is True:
         return -1   # the library reports what does not fit
     if not ok:

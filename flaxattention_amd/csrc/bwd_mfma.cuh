@@ -37,7 +37,10 @@ constexpr int kListBN = 128; // key granularity of the backward tile lists = key
 //               subtraction and applies the scale before dS is rounded
 // p.d_lse2 (optional): the cotangent of the base-2 log-sum-exp output.  d lse / d X_ij = P_ij, so it joins the row
 // term: dX = P o (dP - (delta - log2(e) d_lse2)).
-enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2 };
+//   kBwdDeltaRaw the row sweep of the "unrounded" numerics: delta_i = sum_j P_ij dP_ij with nothing rounded
+//   kBwdHiLo     dQ of the "unrounded" numerics: reads that delta; dP stays in fp32 and dS goes into the product
+//                as a high and a low part (two matrix instructions per fragment); launched with ROUND_S = false
+enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2, kBwdDeltaRaw = 3, kBwdHiLo = 4 };
 template <typename T, int D, int KIND, bool ROUND_S, bool MASKED, int MODE = kBwdFast>
 __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
@@ -89,8 +92,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
     delta = xhalf_sum(dpart);
     if (p.d_lse2) delta -= kLog2e * p.d_lse2[row_id];
     if (q_row < p.Lq && g == 0) delta_out[row_id] = delta;
-  } else if constexpr (MODE == kBwdParity) {
-    delta = delta_out[row_id];  // written by the kBwdDelta launch that precedes this one on the stream
+  } else if constexpr (MODE == kBwdParity || MODE == kBwdHiLo) {
+    delta = delta_out[row_id];  // written by the row-sweep launch that precedes this one on the stream
   }
   float drow = 0.f;  // kBwdDelta: this lane's share of sum_j P_ij round(dP_ij)
   float lse = lse2[row_id];
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   __syncthreads();
   // fast numerics: dP starts at -delta, so the accumulator comes out as dP - delta; the parity numerics
   // round dP first
-  const float neg_delta = MODE == kBwdFast ? -delta : 0.f;
+  const float neg_delta = (MODE == kBwdFast || MODE == kBwdHiLo) ? -delta : 0.f;
   for (int it = 0; it < nt; it++) {
     const int kv0 = t_cur * BN;
     const bool masked = MASKED && ((it >= n_full_t) || (kv0 + BN > p.Lkv));
@@ -229,20 +232,20 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
         asm volatile("" : "+v"(q_opaque), "+v"(kv_opaque));
         mask_block_q(sacc, p.mask, visible, q_opaque, kv_opaque, g, p.Lkv);
       }
-      if constexpr (MODE == kBwdDelta) {
+      if constexpr (MODE == kBwdDelta || MODE == kBwdDeltaRaw) {
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float a0 = dpacc[r], a1 = dpacc[r + 1];
-          round_pair<T>(a0, a1);
+          if constexpr (MODE == kBwdDelta) round_pair<T>(a0, a1);
           drow = fmaf(fast_exp2(sacc[r]), a0, drow);
           drow = fmaf(fast_exp2(sacc[r + 1]), a1, drow);
         }
         continue;
       }
-      vec8 dsf[2];
+      vec8 dsf[2], dsf_lo[2];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
-        typename Pair<T>::v2 pr[4];
+        typename Pair<T>::v2 pr[4], pl[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 8 * tt + 2 * e;
@@ -260,9 +263,11 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
             d1 = fast_exp2(sacc[r + 1]) * dpacc[r + 1];
             if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
           }
-          pr[e] = Pair<T>::pack(d0, d1);
+          if constexpr (MODE == kBwdHiLo) split_pack<T>(d0, d1, pr[e], pl[e]);
+          else pr[e] = Pair<T>::pack(d0, d1);
         }
         dsf[tt] = join_pairs<T>(pr[0], pr[1], pr[2], pr[3]);
+        if constexpr (MODE == kBwdHiLo) dsf_lo[tt] = join_pairs<T>(pl[0], pl[1], pl[2], pl[3]);
       }
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
@@ -271,7 +276,9 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
           const T* ktp = Ks + (32 * nb + 16 * tt) * D;
           short4_t lo = lds_read_tr(ktp + toff[0][db]);
           short4_t hi = lds_read_tr(ktp + toff[1][db]);
-          dqacc[db] = Frag<T>::mfma(join8<vec8>(lo, hi), dsf[tt], dqacc[db]);
+          const vec8 kt = join8<vec8>(lo, hi);
+          dqacc[db] = Frag<T>::mfma(kt, dsf[tt], dqacc[db]);
+          if constexpr (MODE == kBwdHiLo) dqacc[db] = Frag<T>::mfma(kt, dsf_lo[tt], dqacc[db]);
         }
       }
     }
@@ -280,7 +287,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
     __syncthreads();
   }
 
-  if constexpr (MODE == kBwdDelta) {
+  if constexpr (MODE == kBwdDelta || MODE == kBwdDeltaRaw) {
     drow = xhalf_sum(drow);
     if (p.d_lse2) drow -= kLog2e * p.d_lse2[row_id];
     if (q_row < p.Lq && g == 0) delta_out[row_id] = drow;
@@ -320,7 +327,9 @@ template <int D> struct DkvShape {
 // same function the compiler allocates registers differently and the unmasked path runs 5 % slower.
 // PARITY: the numerics of the dense path: dP is rounded through the input dtype before delta (= sum_j P round(dP),
 // from the kBwdDelta sweep) is subtracted, and the scale is applied before dS is rounded.
-template <typename T, int D, int KIND, bool ROUND_S, bool BITS, bool PARITY = false>
+// HILO (the "unrounded" numerics, exclusive with PARITY, launched with ROUND_S = false): P and dS go into their
+// products as a high and a low part each (two matrix instructions per fragment); delta comes from the kBwdDeltaRaw sweep.
+template <typename T, int D, int KIND, bool ROUND_S, bool BITS, bool PARITY = false, bool HILO = false>
 __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dkv_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                                const T* __restrict__ k, const T* __restrict__ v,
                                                                const float* __restrict__ lse2,
@@ -587,10 +596,10 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
         const Mask2 visible(p.mask, b, h, p.Lkv);
         mask_block_kv<BITS>(sacc, p.mask, visible, q_opaque, kv_opaque, p.Lq, p.Lkv);
       }
-      vec8 pf[2], dsf[2];
+      vec8 pf[2], dsf[2], pf_lo[2], dsf_lo[2];
 #pragma unroll
       for (int tt = 0; tt < 2; tt++) {
-        typename Pair<T>::v2 pp[4], dd[4];
+        typename Pair<T>::v2 pp[4], dd[4], pl[4], dl[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           const int r = 8 * tt + 2 * e;
@@ -607,11 +616,20 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
           }
           if (!Score2<KIND>::kGradOne) { d0 *= gacc[r]; d1 *= gacc[r + 1]; }
           if constexpr (PARITY) { d0 *= p.scale; d1 *= p.scale; }
-          pp[e] = Pair<T>::pack(p0, p1);
-          dd[e] = Pair<T>::pack(d0, d1);
+          if constexpr (HILO) {
+            split_pack<T>(p0, p1, pp[e], pl[e]);
+            split_pack<T>(d0, d1, dd[e], dl[e]);
+          } else {
+            pp[e] = Pair<T>::pack(p0, p1);
+            dd[e] = Pair<T>::pack(d0, d1);
+          }
         }
         pf[tt] = join_pairs<T>(pp[0], pp[1], pp[2], pp[3]);
         dsf[tt] = join_pairs<T>(dd[0], dd[1], dd[2], dd[3]);
+        if constexpr (HILO) {
+          pf_lo[tt] = join_pairs<T>(pl[0], pl[1], pl[2], pl[3]);
+          dsf_lo[tt] = join_pairs<T>(dl[0], dl[1], dl[2], dl[3]);
+        }
       }
       // ---- dV^T += dO^T.P, dK^T += Q^T.dS (contraction over this wave's 32 query rows) ----
 #pragma unroll
@@ -625,6 +643,10 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
           }
           dvacc[db] = Frag<T>::mfma(a_do[tt][db], pf[tt], dvacc[db]);
           dkacc[db] = Frag<T>::mfma(a_q[tt][db], dsf[tt], dkacc[db]);
+          if constexpr (HILO) {
+            dvacc[db] = Frag<T>::mfma(a_do[tt][db], pf_lo[tt], dvacc[db]);
+            dkacc[db] = Frag<T>::mfma(a_q[tt][db], dsf_lo[tt], dkacc[db]);
+          }
         }
       }
       }  // query blocks of this wave
@@ -667,16 +689,16 @@ struct BwdArgs {
   hipStream_t s;
 };
 
-template <typename T, int D, int KIND, bool RS, bool BITS, bool PARITY>
+template <typename T, int D, int KIND, bool RS, bool BITS, bool PARITY, bool HILO = false>
 static int launch_dkv_as(const FlexAttnParams& p, const BwdArgs& a) {
   constexpr size_t sm = dkv_smem<D, T>();
   // set on every call: the attribute is per device, and a remembered "already set" would be neither
   // per device nor safe between threads (the call is a host-side table update, no device work)
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS, BITS, PARITY>),
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_dkv_kernel<T, D, KIND, RS, BITS, PARITY, HILO>),
                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)sm) != hipSuccess)
     return 2;
   const int nkt = (p.Lkv + kListBN - 1) / kListBN;
-  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS, BITS, PARITY>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, a.s,
+  hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS, BITS, PARITY, HILO>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, a.s,
                      p, (const T*)a.q, (const T*)a.k, (const T*)a.v, a.lse2, a.delta, (const T*)a.d_o, (T*)a.dk, (T*)a.dv);
   return 0;
 }
@@ -732,8 +754,22 @@ static int launch_parity(const FlexAttnParams& p, const BwdArgs& a) {
   return launch_dkv<T, D, KIND, true, true>(p, a);
 }
 
+// "unrounded" numerics (FLEX_UNROUNDED): unrounded row sweep for delta, then dQ and dK/dV with P and dS carried as
+// high and low parts; S is not rounded
+template <typename T, int D, int KIND>
+static int launch_unrounded(const FlexAttnParams& p, const BwdArgs& a) {
+  if (!(p.flags & FLEX_BWD_ONLY_DKV)) {
+    launch_dq_as<T, D, KIND, false, true, kBwdDeltaRaw>(p, a);
+    launch_dq_as<T, D, KIND, false, true, kBwdHiLo>(p, a);
+  }
+  if (p.flags & FLEX_BWD_ONLY_DQ) return 0;
+  if (p.mask.kind == FLEX_MASK_BITS) return launch_dkv_as<T, D, KIND, false, true, false, true>(p, a);
+  return launch_dkv_as<T, D, KIND, false, false, false, true>(p, a);
+}
+
 template <typename T, int D, int KIND>
 static int launch_rs(const FlexAttnParams& p, const BwdArgs& a) {
+  if (p.flags & FLEX_UNROUNDED) return launch_unrounded<T, D, KIND>(p, a);
   if (p.flags & FLEX_PARITY) return launch_parity<T, D, KIND>(p, a);
   if (p.flags & FLEX_ROUND_S) return launch_one<T, D, KIND, true>(p, a);
   return launch_one<T, D, KIND, false>(p, a);

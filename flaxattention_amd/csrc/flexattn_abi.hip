@@ -80,19 +80,27 @@ extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, in
 // generic kernels apply, FLEX_STRICT is the same numerics.
 static FlexAttnParams with_parity_resolved(const FlexAttnParams* p, bool fused) {
   FlexAttnParams r = *p;
+  if (r.flags & FLEX_UNROUNDED) {
+    r.flags &= ~(FLEX_PARITY | FLEX_ROUND_S | FLEX_STRICT);
+    if (!fused) r.flags &= ~FLEX_UNROUNDED;   // the generic kernels round nothing unless told to
+    return r;
+  }
   if (r.flags & FLEX_PARITY) {
     if (fused) r.flags |= FLEX_ROUND_S;
     else r.flags = (r.flags & ~FLEX_PARITY) | FLEX_STRICT;
   }
   return r;
 }
-static bool wants_fused(const FlexAttnParams* p) { return !(p->flags & (FLEX_FORCE_GENERIC | FLEX_STRICT)); }
+static bool wants_fused(const FlexAttnParams* p) {
+  if (p->flags & FLEX_FORCE_GENERIC) return false;
+  return (p->flags & FLEX_UNROUNDED) || !(p->flags & FLEX_STRICT);
+}
 
 static size_t lse_bytes(const FlexAttnParams* p) { return ((size_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256; }
 
 extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
   // the two passes of the parity numerics hand the log-sum-exp over in lse2, or here when the caller wants no lse2
-  return (p && (p->flags & FLEX_PARITY)) ? lse_bytes(p) : 0;
+  return (p && (p->flags & FLEX_PARITY) && !(p->flags & FLEX_UNROUNDED)) ? lse_bytes(p) : 0;
 }
 
 extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
@@ -180,6 +188,7 @@ extern "C" int flexattn_decode_static(const FlexAttnParams* p, const void* q, co
 
 static int decode_checked(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                           int32_t num_splits, void* workspace, flexattn_stream_t stream) {
+  if (p->flags & FLEX_UNROUNDED) { flex_set_error("flexattn_decode: FLEX_UNROUNDED is served by flexattn_fwd (the decode kernel carries P in one part)"); return 1; }
   if (p->q_index_base < 0 || p->q_index_base % 64 != 0) { flex_set_error("flexattn_decode: q_index_base must be a non-negative multiple of 64 (got %d)", p->q_index_base); return 1; }
   if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
   if (!flex_decode_supported(*p)) {

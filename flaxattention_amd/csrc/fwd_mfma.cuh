@@ -37,7 +37,10 @@ constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dens
 //   kFwdNorm     second pass: P = 2^(x - lse2) is the normalised probability, rounded to the input dtype and
 //                multiplied into V as it is -- what the dense path computes (attention.py:104-105 normalises in
 //                fp32, casts P to the input dtype and then multiplies)
-enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2 };
+//   kFwdHiLo     one pass as kFwdOnePass, but P goes into the P.V product as a high and a low part (two matrix
+//                instructions per fragment) and the row sum adds the unrounded exponentials: the "unrounded"
+//                numerics, launched with ROUND_S = false
+enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2, kFwdHiLo = 3 };
 template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
@@ -237,13 +240,27 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       for (int a = 0; a < RQ; a++) {
         // ---- exponentials; P rounded to the input dtype (not in the log-sum-exp pass, which sums in fp32 what
         // the dense path sums: the unrounded exponentials); l_blk = this lane's share of the block's row sum ----
-        vec8 pf[2];
+        vec8 pf[2], pf_lo[2];
         float l_blk = 0.f;
         auto exponentials = [&](float shift) {
           l_blk = 0.f;
           if constexpr (PASS == kFwdLse) {
 #pragma unroll
             for (int r = 0; r < 16; r++) l_blk += fast_exp2(sacc[a][r] - shift);
+          } else if constexpr (PASS == kFwdHiLo) {
+#pragma unroll
+            for (int tt = 0; tt < 2; tt++) {
+              typename Pair<T>::v2 hi[4], lo[4];
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                const float p0 = fast_exp2(sacc[a][8 * tt + 2 * e] - shift);
+                const float p1 = fast_exp2(sacc[a][8 * tt + 2 * e + 1] - shift);
+                split_pack<T>(p0, p1, hi[e], lo[e]);
+                l_blk += p0 + p1;
+              }
+              pf[tt] = join_pairs<T>(hi[0], hi[1], hi[2], hi[3]);
+              pf_lo[tt] = join_pairs<T>(lo[0], lo[1], lo[2], lo[3]);
+            }
           } else {
 #pragma unroll
             for (int tt = 0; tt < 2; tt++) {
@@ -275,7 +292,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
             const float alpha = fresh ? 1.f : fast_exp2(-delta);
             m_run[a] += delta;
             l_run[a] *= alpha;
-            if constexpr (PASS == kFwdOnePass) {
+            if constexpr (PASS == kFwdOnePass || PASS == kFwdHiLo) {
 #pragma unroll
               for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -290,7 +307,10 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
 #pragma unroll
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int db = 0; db < DB; db++) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+            for (int db = 0; db < DB; db++) {
+              oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
+              if constexpr (PASS == kFwdHiLo) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf_lo[tt], oacc[a][db]);
+            }
         }
       }
       }  // block not entirely hidden
@@ -669,6 +689,12 @@ static void launch_pipe_kernel(const FlexAttnParams& p, const FwdArgs& a) {
 template <typename T, int D, int KIND>
 static void launch_rs(const FlexAttnParams& p, const FwdArgs& a) {
   const bool bits = p.mask.kind == FLEX_MASK_BITS;
+  if (p.flags & FLEX_UNROUNDED) {
+    // "unrounded" numerics: no rounding of S, P carried as a high and a low part
+    if (bits) launch_list_kernel<T, D, KIND, false, true, kFwdHiLo>(p, a);
+    else launch_list_kernel<T, D, KIND, false, false, kFwdHiLo>(p, a);
+    return;
+  }
   if (p.flags & FLEX_PARITY) {
     // parity numerics: a log-sum-exp pass, then the pass that multiplies the normalised, rounded P into V
     // (a.lse2 is never null here: the caller substitutes workspace); S is always rounded through the input dtype

@@ -448,6 +448,14 @@ template <typename T> __device__ __forceinline__ typename Pair<T>::v2 round_pack
   asm("" : "+v"(u));
   return __builtin_bit_cast(typename Pair<T>::v2, u);
 }
+// Split two fp32 values into a high and a low pair of T: hi = T(x), lo = T(x - hi).  A matrix product that is
+// issued once with each pair sees x with twice T's mantissa (16 bits for bf16, 22 for fp16): how the "unrounded"
+// numerics carry P and dS, which the dense path would hold in fp32 if its internal round trips are optimised away.
+template <typename T>
+__device__ __forceinline__ void split_pack(float a, float b, typename Pair<T>::v2& hi, typename Pair<T>::v2& lo) {
+  hi = round_pack<T>(a, b);
+  lo = Pair<T>::pack(a - (float)hi[0], b - (float)hi[1]);
+}
 template <typename T> __device__ __forceinline__ void round_pair(float& a, float& b) {
   typename Pair<T>::v2 h = round_pack<T>(a, b);
   a = (float)h[0];

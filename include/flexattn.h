@@ -105,6 +105,14 @@ enum FlexFlags {
                             Costs about 1.5x the time of the default numerics, which round the
                             unnormalised P and use delta = sum_d O dO.  Where only the generic
                             kernels apply the flag means FLEX_STRICT.  */
+  FLEX_UNROUNDED = 64,   /* fused (MFMA) kernels WITHOUT the dense path's internal round trips: S is not
+                            rounded, P and dS enter their matrix products as a high and a low part of
+                            the input dtype (twice its mantissa), dP stays in fp32 and
+                            delta_i = sum_j P_ij dP_ij comes from an unrounded row sweep; only O, dQ, dK,
+                            dV are rounded.  What the reference computes if XLA's excess-precision
+                            simplification removes the round trips of attention.py:27, 104-105.
+                            Exclusive with FLEX_PARITY / FLEX_ROUND_S (it wins); the generic kernels
+                            do the same when neither FLEX_STRICT nor FLEX_ROUND_S is set.  */
   /* profiling aids for flexattn_bwd: launch only one of the two fused backward
    * kernels.  The dK/dV kernel then reads the delta values a previous complete
    * call left in the same workspace. */

@@ -300,6 +300,32 @@ def test_fused_parity_numerics_f16(dev, D, name, score, oscore):
         strict=False, opts={"numerics": "parity"}, scale_maxabs=big)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name,score,oscore", SCORES, ids=[s[0] for s in SCORES])
+def test_fused_unrounded_numerics(dev, dtype, D, name, score, oscore):
+    """kernel_options={"numerics": "unrounded"}: no internal round trip (S unrounded, P and dS carried as high and low
+    parts, delta from an unrounded row sweep).  Held to the stated tolerance against the oracle WITHOUT the dense
+    path's round trips (strict=False), the variant an XLA build that optimises them away would compute."""
+    print(f"case fused unrounded {name} {dtype} D{D}", flush=True)
+    B, Hq, Hkv, Lq, Lkv = 2, 4, 2, 256, 320
+    q, k, v = seeded_qkv(B, Hq, Hkv, Lq, Lkv, D, dtype)
+    d_o = torch.randn((B, Hq, Lq, D), generator=torch.Generator().manual_seed(3)).to(dtype)
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    bm = fa.create_block_mask(causal_mask, B, Hq, Lq, Lkv, device=dev)
+    out, lse = fa.flax_attention(qd, kd, vd, score_mod=score, block_mask=bm, enable_gqa=True, return_lse=True,
+                                 kernel_options={"numerics": "unrounded"})
+    out.backward(d_o.to(dev))
+    want, want_lse = ref_attention(q, k, v, oscore, o_causal_mask, strict=False, return_lse=True)
+    wq, wk, wv = ref_attention_bwd(q, k, v, d_o, oscore, o_causal_mask, strict=False)
+    big = name == "alibi_ref"
+    close(out, want, dtype, "O")
+    assert max_abs(lse.detach().cpu(), want_lse) <= 2e-2
+    close(qd.grad, wq, dtype, "dQ", scale_maxabs=big)
+    close(kd.grad, wk, dtype, "dK", scale_maxabs=big)
+    close(vd.grad, wv, dtype, "dV", scale_maxabs=big)
+
+
 def test_parity_numerics_dense_no_lists(dev):
     """Parity numerics without a mask (no tile lists, every tile visited) and with a ragged key length."""
     for dtype in (torch.bfloat16, torch.float16):
