@@ -55,9 +55,13 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
   constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor
   // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled
-  // rows): while one tile is consumed the next one lands, one workgroup barrier per tile
-  __shared__ __align__(16) T Ksm[2][BN * D];
-  __shared__ __align__(16) T Vsm[2][BN * D];
+  // rows): while one tile is consumed the next one lands, one workgroup barrier per tile.  Each stage is a
+  // variable of its own and every access names its stage at compile time (the tile loop is unrolled by two):
+  // only then can the compiler tell that a read of one stage need not wait for the fetch into the other.
+  __shared__ __align__(16) T Ksm0[BN * D];
+  __shared__ __align__(16) T Ksm1[BN * D];
+  __shared__ __align__(16) T Vsm0[BN * D];
+  __shared__ __align__(16) T Vsm1[BN * D];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -105,8 +109,8 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   int n_full, n_part = 0;
   if (tl.kv_num) {
     const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
-    n_full = tl.full_kv_num[row];
-    n_part = tl.kv_num[row];
+    n_full = uniform_ld(tl.full_kv_num + row);
+    n_part = uniform_ld(tl.kv_num + row);
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
     part_idx = tl.kv_idx + row * tl.n_kv_blocks;
   } else {
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   auto tile_at = [&](int it) -> int {
     if (!full_idx) return it;
     const int e = sub == 2 ? (it >> 1) : it, part = sub == 2 ? (it & 1) : 0;
-    return (e < n_full ? full_idx[e] : part_idx[e - n_full]) * sub + part;
+    return uniform_ld(e < n_full ? full_idx + e : part_idx + (e - n_full)) * sub + part;
   };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
@@ -131,19 +135,48 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
   // tile fetch: wave w fills rows [32w, 32w + 32) of the K and the V tile, RPI rows per instruction;
   // the lane that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
   const int fill_row = lane / CPR, fill_pos = lane % CPR;
-  auto issue_tile = [&](int stage, int kv0) {
-    const int lim = p.Lkv - 1 - kv0;  // rows past the end: clamped (finite filler, masked out below)
+  // the per-lane part of a fetch address (row among the 16 of a swizzle period, swizzled chunk) is the same for
+  // every tile: kept as byte offsets from a wave-uniform row address
+  const int wu = __builtin_amdgcn_readfirstlane(w);
+  constexpr int NP = 16 / RPI;  // fetch instructions per swizzle period
+  uint32_t koff[NP], voff[NP];
 #pragma unroll
-    for (int j = 0; j < NI; j++) {
-      const int r0 = (BN / 4) * w + RPI * j;
-      const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);  // the wave's first row is a multiple of 16
-      const int row = min(r0 + fill_row, lim);
-      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
-      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
-                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
+  for (int jp = 0; jp < NP; jp++) {
+    const int row = RPI * jp + fill_row;
+    const int chunk = fill_pos ^ lds_swz<D>(row);  // the wave's first row is a multiple of 16
+    koff[jp] = (uint32_t)((row * ks2 + chunk * 8) * (int64_t)sizeof(T));
+    voff[jp] = (uint32_t)((row * vs2 + chunk * 8) * (int64_t)sizeof(T));
+  }
+  auto issue_tile = [&](auto stage, int kv0_in) {
+    T* const Kst = stage_ptr(stage, Ksm0, Ksm1);
+    T* const Vst = stage_ptr(stage, Vsm0, Vsm1);
+    const int kv0 = __builtin_amdgcn_readfirstlane(kv0_in);
+    const int lim = p.Lkv - 1 - kv0;
+    if (lim >= BN - 1) {
+#pragma unroll
+      for (int j = 0; j < NI; j++) {
+        const int r0 = (BN / 4) * wu + RPI * (j - j % NP);
+        const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)(kv0 + r0) * ks2);
+        const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)(kv0 + r0) * vs2);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt + koff[j % NP]),
+                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * (j % NP)) * D), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt + voff[j % NP]),
+                                         (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * (j % NP)) * D), 16, 0, 0);
+      }
+    } else {
+      // the last tile of a ragged length: rows past the end are clamped (finite filler, masked out below)
+#pragma unroll
+      for (int j = 0; j < NI; j++) {
+        const int r0 = (BN / 4) * wu + RPI * j;
+        const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);
+        const int row = min(r0 + fill_row, lim);
+        const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
+        const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                         (__attribute__((address_space(3))) void*)(Vst + r0 * D), 16, 0, 0);
+      }
     }
   };
   // element offsets inside a 32-row block: row fragments (row i32, chunk 2s + g sits at (2s) ^ kz) and
@@ -172,21 +205,23 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
 
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
-  if (nt > 0) issue_tile(0, t_cur * BN);
+  if (nt > 0) issue_tile(StageC<0>{}, t_cur * BN);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   // fast numerics: dP starts at -delta, so the accumulator comes out as dP - delta; the parity numerics
   // round dP first
   const float neg_delta = (MODE == kBwdFast || MODE == kBwdHiLo) ? -delta : 0.f;
-  for (int it = 0; it < nt; it++) {
+  // one tile out of the stage named by `stage` (= it & 1)
+  auto tile_step = [&](auto stage, int it) {
+    constexpr int ST = decltype(stage)::value;
     const int kv0 = t_cur * BN;
     const bool masked = MASKED && ((it >= n_full_t) || (kv0 + BN > p.Lkv));
-    const T* Ks = Ksm[it & 1];
-    const T* Vs = Vsm[it & 1];
+    const T* const Ks = stage_ptr(stage, Ksm0, Ksm1);
+    const T* const Vs = stage_ptr(stage, Vsm0, Vsm1);
     if (it + 1 < nt) {
       // the other stage was last read before the previous barrier: the next tile lands there
       // while this one is consumed; the tile index after that is looked up a tile ahead
-      issue_tile((it + 1) & 1, t_nxt * BN);
+      issue_tile(StageC<1 - ST>{}, t_nxt * BN);
       t_cur = t_nxt;
       if (it + 2 < nt) t_nxt = tile_at(it + 2);
     }
@@ -285,6 +320,10 @@ __global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const 
     // this wave's share of the next tile has landed; after the barrier everyone's has
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+  };
+  for (int it = 0; it < nt; it += 2) {
+    tile_step(StageC<0>{}, it);
+    if (it + 1 < nt) tile_step(StageC<1>{}, it + 1);
   }
 
   if constexpr (MODE == kBwdDelta || MODE == kBwdDeltaRaw) {
@@ -405,8 +444,8 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
     int n_full, n_part = 0;
     if (tl.kv_num) {
       const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_kv_blocks + kt;
-      n_full = tl.full_q_num[row];
-      n_part = tl.q_num[row];
+      n_full = uniform_ld(tl.full_q_num + row);
+      n_part = uniform_ld(tl.q_num + row);
       full_idx = tl.full_q_idx + row * tl.n_q_blocks;
       part_idx = tl.q_idx + row * tl.n_q_blocks;
     } else {
@@ -421,7 +460,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 
     auto tile_at = [&](int it) -> int {
       if (!full_idx) return it;
-      return it < n_full ? full_idx[it] : part_idx[it - n_full];
+      return uniform_ld(it < n_full ? full_idx + it : part_idx + (it - n_full));
     };
     u32x4 qreg[DIRECT ? 1 : NLD], oreg[DIRECT ? 1 : NLD];
     float lreg = INFINITY, dreg = 0.f;

@@ -92,8 +92,8 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
     steps_total = kv_last >= vis_lo_any ? kv_last / kStep - step_lo + 1 : 0;
   } else if (tl.kv_num && G == 1 && tl.kv_block == 2 * kStep && p.q_index_base % tl.q_block + p.Lq <= tl.q_block) {
     const int64_t row = (b * tl.stride_b + hk * tl.stride_h) * tl.n_q_blocks + p.q_index_base / tl.q_block;
-    n_full = tl.full_kv_num[row];
-    const int n_part = tl.kv_num[row];
+    n_full = uniform_ld(tl.full_kv_num + row);
+    const int n_part = uniform_ld(tl.kv_num + row);
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
     part_idx = tl.kv_idx + row * tl.n_kv_blocks;
     steps_total = 2 * (n_full + n_part);
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1
   auto step_kv0 = [&](int st) -> int {
     if (!full_idx) return (step_lo + st) * kStep;
     const int item = st >> 1;
-    const int tile = item < n_full ? full_idx[item] : part_idx[item - n_full];
+    const int tile = uniform_ld(item < n_full ? full_idx + item : part_idx + (item - n_full));
     return tile * (2 * kStep) + (st & 1) * kStep;
   };
   const int per = (steps_total + splits - 1) / splits;

@@ -86,8 +86,8 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   int n_full, n_part = 0;
   if (tl.kv_num) {
     const int64_t row = (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt;
-    n_full = tl.full_kv_num[row];
-    n_part = tl.kv_num[row];
+    n_full = uniform_ld(tl.full_kv_num + row);
+    n_part = uniform_ld(tl.kv_num + row);
     full_idx = tl.full_kv_idx + row * tl.n_kv_blocks;
     part_idx = tl.kv_idx + row * tl.n_kv_blocks;
   } else {
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   const int nt = n_full + n_part;
   auto tile_at = [&](int it) -> int {
     if (!full_idx) return nt - 1 - it;
-    return it < n_part ? part_idx[n_part - 1 - it] : full_idx[n_full - 1 - (it - n_part)];
+    return uniform_ld(it < n_part ? part_idx + (n_part - 1 - it) : full_idx + (n_full - 1 - (it - n_part)));
   };
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
@@ -109,13 +109,33 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
   u32x4 kreg[NLD], vreg[NLD];
-  auto load_tile = [&](int kv0) {
+  // the per-lane part of a load address (row inside the tile, chunk) is the same for every tile: kept as byte
+  // offsets from the tile's first row, whose address is wave-uniform
+  uint32_t klo[NLD], vlo[NLD];
 #pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
-      kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
-      if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+  for (int j = 0; j < NLD; j++) {
+    const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+    klo[j] = (uint32_t)((r * ks2 + cc * 8) * (int64_t)sizeof(T));
+    vlo[j] = (uint32_t)((r * vs2 + cc * 8) * (int64_t)sizeof(T));
+  }
+  auto load_tile = [&](int kv0_in) {
+    const int kv0 = __builtin_amdgcn_readfirstlane(kv0_in);
+    if (kv0 + BN <= p.Lkv) {
+      const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)kv0 * ks2);
+      const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)kv0 * vs2);
+#pragma unroll
+      for (int j = 0; j < NLD; j++) {
+        kreg[j] = *reinterpret_cast<const u32x4*>(kt + klo[j]);
+        if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vt + vlo[j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NLD; j++) {
+        const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
+        const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
+        kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
+        if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+      }
     }
   };
   auto store_tile = [&](int stage) {
@@ -383,8 +403,15 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   // transposing reads conflict-free.  The lane that fills position (r, pos) therefore fetches
   // chunk pos ^ lds_swz(r) of that row.
   constexpr int kTileElems = BN * D;  // 8 KB per tile
-  __shared__ __align__(16) T Ksm[3][kTileElems];
-  __shared__ __align__(16) T Vsm[3][kTileElems];
+  // each stage is a variable of its own and every access names its stage at compile time (the tile loop is
+  // unrolled by three): only then can the compiler tell that a read of one stage need not wait for the fetch
+  // into another
+  __shared__ __align__(16) T Ksm0[kTileElems];
+  __shared__ __align__(16) T Ksm1[kTileElems];
+  __shared__ __align__(16) T Ksm2[kTileElems];
+  __shared__ __align__(16) T Vsm0[kTileElems];
+  __shared__ __align__(16) T Vsm1[kTileElems];
+  __shared__ __align__(16) T Vsm2[kTileElems];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -416,19 +443,46 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
 
   // ---- tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, 8 rows per instruction ----
   const int fill_row = lane >> 3;                         // row inside the 8-row group
-  auto issue_tile = [&](int stage, int kv0) {
-    const int lim = p.Lkv - 1 - kv0;  // rows past the end are clamped (finite filler, masked out below)
+  // the per-lane part of a fetch address (row among the wave's 16, swizzled chunk) is the same for every tile:
+  // kept as byte offsets from the wave's first row of the tile, whose address is wave-uniform
+  const int wu = __builtin_amdgcn_readfirstlane(w);
+  uint32_t kfo[2], vfo[2];
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-      const int r0 = 16 * w + 8 * j;
-      const int fill_chunk = (lane & 7) ^ lds_swz<D>(8 * j + fill_row);  // logical chunk this lane fetches
-      const int row = min(r0 + fill_row, lim);
-      const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + fill_chunk * 8;
-      const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + fill_chunk * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
-                                       (__attribute__((address_space(3))) void*)(Ksm[stage] + r0 * D), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                       (__attribute__((address_space(3))) void*)(Vsm[stage] + r0 * D), 16, 0, 0);
+  for (int j = 0; j < 2; j++) {
+    const int row = 8 * j + fill_row;
+    const int fill_chunk = (lane & 7) ^ lds_swz<D>(row);  // logical chunk this lane fetches
+    kfo[j] = (uint32_t)((row * ks2 + fill_chunk * 8) * (int64_t)sizeof(T));
+    vfo[j] = (uint32_t)((row * vs2 + fill_chunk * 8) * (int64_t)sizeof(T));
+  }
+  auto issue_tile = [&](auto stage, int kv0) {
+    T* const Kst = stage_ptr(stage, Ksm0, Ksm1, Ksm2);
+    T* const Vst = stage_ptr(stage, Vsm0, Vsm1, Vsm2);
+    const int lim = p.Lkv - 1 - kv0;
+    if (!TAIL || lim >= BN - 1) {
+      const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)(kv0 + 16 * wu) * ks2);
+      const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)(kv0 + 16 * wu) * vs2);
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int r0 = 16 * wu + 8 * j;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt + kfo[j]),
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt + vfo[j]),
+                                         (__attribute__((address_space(3))) void*)(Vst + r0 * D), 16, 0, 0);
+      }
+    } else {
+      // the last tile of a ragged length: rows past the end are clamped (finite filler, masked out below)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int r0 = 16 * wu + 8 * j;
+        const int fill_chunk = (lane & 7) ^ lds_swz<D>(8 * j + fill_row);
+        const int row = min(r0 + fill_row, lim);
+        const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + fill_chunk * 8;
+        const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + fill_chunk * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                         (__attribute__((address_space(3))) void*)(Vst + r0 * D), 16, 0, 0);
+      }
     }
   };
   // ---- fragment reads ----
@@ -492,31 +546,31 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;   // tile it + 1
   int t_nx2 = nt > 2 ? tile_at(2) : 0;   // tile it + 2
-  if (nt > 0) issue_tile(0, t_cur * BN);
-  if (nt > 1) issue_tile(1, t_nxt * BN);
+  if (nt > 0) issue_tile(StageC<0>{}, t_cur * BN);
+  if (nt > 1) issue_tile(StageC<1>{}, t_nxt * BN);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   // S of the first unit
-  read_k(Ksm[0], 0);
+  read_k(Ksm0, 0);
 #pragma unroll
   for (int r = 0; r < 16; r++) s_cur[r] = 0.f;
 #pragma unroll
   for (int s = 0; s < DS; s++) s_cur = Frag<T>::mfma(kfr[s], qf[0][s], s_cur);
 
   const int slot = blockIdx.x >= (gridDim.x >> 1) ? 1 : 0;  // second half of the grid = second workgroup of a compute unit
-  int st = 0;  // LDS stage of the current tile (it % 3)
-  for (int it = 0; it < nt; it++) {
+  // one tile out of the stage named by `stage` (= it % 3)
+  auto tile_step = [&](auto stage, int it) {
+    constexpr int ST = decltype(stage)::value;
     // Two workgroups share a compute unit and the instruction arbiter favours the older wave,
     // which leaves the younger one behind until it runs alone at the end.  All workgroups have
     // the same amount of work here, so trading the wave priority between them every tile keeps
     // both advancing at the same pace.
     if ((it ^ slot) & 1) __builtin_amdgcn_s_setprio(2); else __builtin_amdgcn_s_setprio(0);
     const int kv0 = t_cur * BN;
-    const int st_n = st == 2 ? 0 : st + 1;
-    const T* Ks = Ksm[st];
-    const T* Vs = Vsm[st];
-    const T* Kn = Ksm[st_n];
-    const int st_p = st == 0 ? 2 : st - 1;  // stage of the previous tile = stage of tile it + 2
+    const T* const Ks = stage_ptr(stage, Ksm0, Ksm1, Ksm2);
+    const T* const Vs = stage_ptr(stage, Vsm0, Vsm1, Vsm2);
+    const T* const Kn = stage_ptr(StageC<(ST + 1) % 3>{}, Ksm0, Ksm1, Ksm2);
+    const StageC<(ST + 2) % 3> st_p;  // stage of the previous tile = stage of tile it + 2
     const int kv_nx2 = t_nx2 * BN;
     t_cur = t_nxt;
     t_nxt = t_nx2;
@@ -634,7 +688,13 @@ __global__ __launch_bounds__(256, 2) void fwd_pipe_kernel(FlexAttnParams p, cons
         s_cur = s_nxt;
       }
     }
-    st = st_n;
+  };
+  for (int it = 0; it < nt; it += 3) {
+    tile_step(StageC<0>{}, it);
+    if (it + 1 < nt) {  // nested: no path may reach a stage's step without the step before it
+      tile_step(StageC<1>{}, it + 1);
+      if (it + 2 < nt) tile_step(StageC<2>{}, it + 2);
+    }
   }
   __builtin_amdgcn_s_setprio(0);
   // the last unit's P is still pending

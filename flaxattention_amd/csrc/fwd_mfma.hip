@@ -9,7 +9,8 @@ int flex_mfma_fwd_f16_128(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_128(const FlexAttnParams& p, const FwdArgs& a);
 
-static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0; }
+// rows of 16-byte chunks; the kernels keep the offset of a row inside a tile in 32 bits
+static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && s[2] >= 0 && s[2] < (1 << 24); }
 
 // dtype / head size / layout the MFMA kernels can take at all
 bool flex_mfma_shape_ok(const FlexAttnParams& p) {

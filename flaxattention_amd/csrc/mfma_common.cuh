@@ -495,6 +495,22 @@ __device__ __forceinline__ float tile_max(const float16_t (&x)[2]) {
   return max3(max3(a, b, x[0][15]), x[1][15], x[1][15]);
 }
 
+// LDS stages as separate variables, selected at compile time: the compiler tracks a direct global -> LDS fetch per
+// variable, so a read of one stage does not wait for a fetch into another only if every access names its
+// variable statically.
+template <int S> struct StageC { static constexpr int value = S; };
+template <int S, typename P> __device__ __forceinline__ P* stage_ptr(StageC<S>, P* s0, P* s1) { return S == 0 ? s0 : s1; }
+template <int S, typename P> __device__ __forceinline__ P* stage_ptr(StageC<S>, P* s0, P* s1, P* s2) {
+  return S == 0 ? s0 : (S == 1 ? s1 : s2);
+}
+
+// Tile-list entries (written by an earlier launch, never by these kernels) are read through the constant
+// address space: the entry lands in a scalar register, the addresses derived from it stay wave-uniform, and
+// waiting for it does not wait for the vector loads in flight.
+__device__ __forceinline__ int uniform_ld(const int32_t* ptr) {
+  return *(const __attribute__((address_space(4))) int32_t*)ptr;
+}
+
 // Unpadded LDS tiles (rows of 2D bytes, so that a wave-wide direct global -> LDS load can fill 1 KB
 // of consecutive rows): the 16-byte chunk c of row r is kept at chunk position c ^ lds_swz<D>(r),
 // a function of r & 15 chosen so that both kinds of operand reads are free of bank conflicts
