@@ -1,6 +1,6 @@
 """MI355X-native FlexAttention with the Python surface of flaxattention
 (flaxattention/__init__.py:1-22)."""
-from .core.attention import math_attention, flax_attention, flax_attention_pallas
+from .core.attention import math_attention, flax_attention, flax_attention_pallas, kernel_family
 from .core.blockmask import BlockMask, create_block_mask, create_mask, and_masks, or_masks, noop_mask
 from .core.common import _mask_mod_signature, _score_mod_signature, MaskMod, ScoreMod
 from .utils import visualize_attention_scores
@@ -22,4 +22,5 @@ __all__ = [
     "MaskMod",
     "ScoreMod",
     "FlexAttnError",
+    "kernel_family",
 ]

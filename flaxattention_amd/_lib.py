@@ -62,7 +62,7 @@ class FlexAttnParams(C.Structure):
 
 
 EXPORTS = [
-    "flexattn_abi_version", "flexattn_last_error", "flexattn_preferred_tiles",
+    "flexattn_abi_version", "flexattn_last_error", "flexattn_preferred_tiles", "flexattn_kernel_family",
     "flexattn_block_mask_workspace_bytes", "flexattn_block_mask_build",
     "flexattn_fwd_workspace_bytes", "flexattn_fwd",
     "flexattn_bwd_workspace_bytes", "flexattn_bwd",
@@ -98,6 +98,7 @@ def lib() -> C.CDLL:
     L.flexattn_abi_version.restype = C.c_int
     L.flexattn_last_error.restype = C.c_char_p
     L.flexattn_preferred_tiles.argtypes = [C.c_int32] * 6 + [C.POINTER(C.c_int32)] * 2
+    L.flexattn_kernel_family.argtypes = [C.POINTER(FlexAttnParams), C.c_int32]
     L.flexattn_block_mask_workspace_bytes.restype = C.c_size_t
     L.flexattn_block_mask_workspace_bytes.argtypes = [C.c_int32] * 4
     L.flexattn_block_mask_build.argtypes = ([C.POINTER(FlexMask)] + [C.c_int32] * 6 +

@@ -39,7 +39,7 @@ selects numerics here:
                           whenever it applies (fp16/bf16, D = Dv in {64, 128},
                           at most 64 query rows per KV head, at least 512 keys)
     {"decode_splits": n}  force the split-KV decode kernel with n splits
-    {"pad_head_dim": bool}  16-bit inputs whose head sizes are not D = Dv in {64, 128} (but at most
+    {"pad_head_dim": bool}  inputs whose head sizes are not D = Dv in {64, 128} (but at most
                           128) are zero-padded to the next of those so that the fused kernels serve
                           them (default True)
     {"tile_lists": bool}  False: call the library without tile lists, as a C-ABI caller without a
@@ -446,14 +446,14 @@ def _as_kernel_layout(t: Array) -> Array:
 
 
 def _pad_head_dims(q: Array, k: Array, v: Array, kernel_options) -> Tuple[Array, Array, Array]:
-    """The fused kernels exist for D = Dv in {64, 128}.  Other head sizes up to 128 (and Dv < D) of
-    16-bit inputs are zero-padded to the next of those: zero feature columns add nothing to Q.K^T, the
+    """The matrix-core kernels (16-bit and float32) exist for D = Dv in {64, 128}.  Other head sizes up to 128
+    (and Dv < D) are zero-padded to the next of those: zero feature columns add nothing to Q.K^T, the
     padded columns of O are dropped by the caller and the padded columns of the gradients are cut off by
     autograd, so the result is the one of the original problem at matrix-core speed.  Opt out with
     kernel_options={"pad_head_dim": False}; the faithful and the generic kernels take any size as it is."""
     opts = kernel_options or {}
     D, Dv = q.shape[-1], v.shape[-1]
-    if (q.dtype not in (torch.float16, torch.bfloat16) or opts.get("strict", False)
+    if (q.dtype not in (torch.float16, torch.bfloat16, torch.float32) or opts.get("strict", False)
             or opts.get("backend", "auto") == "generic" or not opts.get("pad_head_dim", True)):
         return q, k, v
     Dp = 64 if max(D, Dv) <= 64 else 128
@@ -532,6 +532,36 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
     if return_lse:
         return out, lse2 * math.log(2.0)
     return out
+
+
+_FAMILIES = {0: "generic", 1: "mfma_16bit", 2: "mfma_f32"}
+
+
+def kernel_family(query: Array, key: Array, value: Array, score_mod: Optional[_score_mod_signature] = None,
+                  block_mask: Optional[BlockMask] = None, scale: Optional[float] = None,
+                  kernel_options: Optional[Dict[str, Any]] = None, backward: bool = False) -> str:
+    """Which kernels flax_attention runs for these inputs: "generic" (vector ALU), "mfma_16bit" or "mfma_f32"
+    (matrix cores).  Asks the library (flexattn_kernel_family) with the parameters the call itself would pass;
+    nothing is computed.  No counterpart in the reference, which has one dense path (core/attention.py:14-106)."""
+    _require_device(query, key, value)
+    if score_mod is None:
+        score_mod = _identity
+    if block_mask is None:
+        block_mask = _create_empty_block_mask(query, key)
+    if scale is None:
+        scale = 1.0 / math.sqrt(query.shape[-1])
+    q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
+    try:
+        plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
+    except ScoreModNotLowered:
+        # linearised at the scores of the call: dense multiplicative and additive tables (FLEX_SCORE_AFFINE)
+        opts = dict(kernel_options or {})
+        opts["tile_lists"] = opts.get("tile_lists", True)
+        plan = _make_plan(q, k, v, _identity, block_mask, None, scale, opts)
+        plan.score = ScoreMod(_lib.SCORE_AFFINE, mul=torch.ones(1, device=q.device), add=None)
+    o_like = torch.empty((q.shape[0], q.shape[1], q.shape[2], v.shape[3]), dtype=q.dtype, device="meta")
+    p = plan.params(q, k, v, o_like)
+    return _FAMILIES[_lib.lib().flexattn_kernel_family(_lib.C.byref(p), 1 if backward else 0)]
 
 
 def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Optional[_score_mod_signature] = None,

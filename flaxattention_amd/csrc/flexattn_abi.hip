@@ -30,6 +30,10 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
                        void* workspace, hipStream_t s);
 void* flex_decode_static_scratch(size_t* bytes);
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb);
+bool flex_f32_mfma_supported(const FlexAttnParams& p, int which);
+int flex_f32_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+int flex_f32_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                      const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
 
 static int validate(const FlexAttnParams* p, const char* who) {
   if (!p) { flex_set_error("%s: null params", who); return 1; }
@@ -65,7 +69,7 @@ static int check_launch(const char* who) {
   return 0;
 }
 
-extern "C" int flexattn_abi_version(void) { return 3; }
+extern "C" int flexattn_abi_version(void) { return 4; }
 extern "C" const char* flexattn_last_error(void) { return g_err; }
 
 extern "C" int flexattn_preferred_tiles(int32_t dtype, int32_t D, int32_t Dv, int32_t Lq, int32_t Lkv, int32_t which, int32_t* qb, int32_t* kvb) {
@@ -96,6 +100,13 @@ static bool wants_fused(const FlexAttnParams* p) {
   return (p->flags & FLEX_UNROUNDED) || !(p->flags & FLEX_STRICT);
 }
 
+extern "C" int flexattn_kernel_family(const FlexAttnParams* p, int32_t which) {
+  if (!p || !wants_fused(p)) return FLEX_FAMILY_GENERIC;
+  if (flex_f32_mfma_supported(*p, which ? 1 : 0)) return FLEX_FAMILY_MFMA_F32;
+  if (which ? flex_mfma_bwd_supported(*p) : flex_mfma_fwd_supported(*p)) return FLEX_FAMILY_MFMA_16BIT;
+  return FLEX_FAMILY_GENERIC;
+}
+
 static size_t lse_bytes(const FlexAttnParams* p) { return ((size_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256; }
 
 extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
@@ -110,6 +121,12 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o) { flex_set_error("flexattn_fwd: null tensor pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
+  // float32 inputs: the reference rounds nothing below fp32, so every numerics mode but FLEX_STRICT is the same
+  // computation and runs on the matrix cores
+  if (wants_fused(p) && flex_f32_mfma_supported(*p, 0)) {
+    if (int rc32 = flex_f32_mfma_fwd(*p, q, k, v, o, lse2, s)) return rc32;
+    return check_launch("flexattn_fwd");
+  }
   const bool fused = wants_fused(p) && flex_mfma_fwd_supported(*p);
   const FlexAttnParams pr = with_parity_resolved(p, fused);
   if (fused) {
@@ -142,6 +159,10 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o || !lse2 || !d_o || !dq || !dk || !dv || !workspace) { flex_set_error("flexattn_bwd: null pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
+  if (wants_fused(p) && flex_f32_mfma_supported(*p, 1)) {
+    if (int rc32 = flex_f32_mfma_bwd(*p, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s)) return rc32;
+    return check_launch("flexattn_bwd");
+  }
   const bool fused = wants_fused(p) && flex_mfma_bwd_supported(*p);
   const FlexAttnParams pr = with_parity_resolved(p, fused);
   if (fused) rc = flex_mfma_bwd(pr, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s);

@@ -168,6 +168,17 @@ typedef struct FlexAttnParams {
 int flexattn_abi_version(void);
 const char* flexattn_last_error(void);
 
+/* Which kernel family flexattn_fwd (which = 0) or flexattn_bwd (which = 1) runs for these parameters: a pure
+ * function of *p, no device work.  The reference has one dense path and one fused kernel
+ * (core/attention.py:14-106, kernel/attention.py:166-653); here the choice depends on dtype, head sizes, strides,
+ * flags and list granularity, and a caller (or a test) can ask instead of guessing. */
+enum FlexKernelFamily {
+  FLEX_FAMILY_GENERIC = 0,    /* vector-ALU kernels: any dtype / head size, FLEX_STRICT numerics */
+  FLEX_FAMILY_MFMA_16BIT = 1, /* fused fp16 / bf16 matrix-core kernels */
+  FLEX_FAMILY_MFMA_F32 = 2    /* fp32 matrix-core kernels */
+};
+int flexattn_kernel_family(const FlexAttnParams* p, int32_t which);
+
 /* Tile sizes the fused kernels want their FlexTileLists built at for this
  * problem (0/0 when only the generic kernels apply and lists are ignored).
  * which = 0: FlexAttnParams.tiles (forward, decode); which = 1: tiles_bwd. */

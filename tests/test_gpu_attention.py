@@ -140,6 +140,82 @@ def test_config1_fp32_causal(dev):
     run(dev, torch.float32, 1, 4, 4, 256, 256, 64, mask=causal_mask, omask=o_causal_mask)
 
 
+# ---- float32 on the matrix cores: what float32 inputs run on unless kernel_options["strict"] is set ----
+def family(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, mask=None, backward=False, opts=None):
+    q = torch.zeros((B, Hq, Lq, D), dtype=dtype, device=dev)
+    k = torch.zeros((B, Hkv, Lkv, D), dtype=dtype, device=dev)
+    bm = fa.create_block_mask(mask, B, Hq, Lq, Lkv, device=dev) if mask is not None else None
+    return fa.kernel_family(q, k, k, block_mask=bm, kernel_options=opts, backward=backward)
+
+
+def test_kernel_family_query(dev):
+    for bwd in (False, True):
+        assert family(dev, torch.float32, 1, 4, 4, 256, 256, 64, causal_mask, bwd) == "mfma_f32"
+        assert family(dev, torch.float32, 1, 4, 4, 256, 256, 32, causal_mask, bwd) == "mfma_f32"   # zero-padded to 64
+        assert family(dev, torch.float32, 1, 4, 4, 256, 256, 64, causal_mask, bwd, {"strict": True}) == "generic"
+        assert family(dev, torch.float32, 1, 4, 4, 256, 256, 256, None, bwd) == "generic"
+        assert family(dev, torch.float16, 1, 4, 4, 256, 256, 64, causal_mask, bwd) == "mfma_16bit"
+        assert family(dev, torch.bfloat16, 1, 4, 2, 100, 300, 128, None, bwd) == "mfma_16bit"
+        assert family(dev, torch.bfloat16, 1, 4, 4, 256, 256, 64, None, bwd, {"backend": "generic"}) == "generic"
+
+
+SCORES_F32 = [
+    ("identity", None, None),
+    ("checker_diff", checkerboard, o_checkerboard),
+    ("checker_kv", generate_checkerboard(2.0, 0.5, "kv"), o_checkerboard_kv),
+    ("alibi_cfg", generate_alibi_bias(4, sign=-1.0), o_alibi_config(4)),
+    ("softcap", generate_tanh_softcap(5.0), o_tanh_softcap(5.0)),
+    ("relbias", generate_rel_bias(0.03), o_rel_bias(0.03)),
+]
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("name,score,oscore", SCORES_F32, ids=[s[0] for s in SCORES_F32])
+def test_fp32_mfma_scores(dev, D, name, score, oscore):
+    print(f"case fp32 mfma {name} D{D}", flush=True)
+    run(dev, torch.float32, 2, 4, 4, 192, 256, D, score=score, oscore=oscore, mask=causal_mask, omask=o_causal_mask,
+        strict=False)
+
+
+MASKS_F32 = [
+    ("window", generate_sliding_window(40), o_sliding_window(40)),
+    ("sink", generate_attention_sink(50, 4), o_attention_sink(50, 4)),
+    ("sink_lt", generate_attention_sink(50, 3), o_sink_window_lt(50, 4)),
+    ("offset", offset_causal_mask(64), o_offset_causal(64)),
+]
+
+
+@pytest.mark.parametrize("name,mask,omask", MASKS_F32, ids=[m[0] for m in MASKS_F32])
+def test_fp32_mfma_masks(dev, name, mask, omask):
+    print(f"case fp32 mfma mask {name}", flush=True)
+    run(dev, torch.float32, 1, 2, 2, 300, 450, 64, mask=mask, omask=omask, strict=False)
+
+
+def test_fp32_mfma_config1(dev):
+    """Benchmark configuration 1 on the path float32 takes by default."""
+    run(dev, torch.float32, 1, 4, 4, 256, 256, 64, mask=causal_mask, omask=o_causal_mask, strict=False)
+
+
+def test_fp32_mfma_bitmap_mask_and_dead_rows(dev):
+    def weird(b, h, q_idx, kv_idx):
+        return ((q_idx * 7 + kv_idx * 3 + h) % 11 < 6) & (q_idx % 5 != 0)
+    run(dev, torch.float32, 2, 3, 3, 100, 150, 32, mask=weird, omask=weird, strict=False)
+
+
+def test_fp32_mfma_gqa_ragged_no_lists(dev):
+    run(dev, torch.float32, 2, 8, 2, 77, 203, 64, Dv=32, mask=causal_mask, omask=o_causal_mask,
+        score=generate_alibi_bias(8, -1.0), oscore=o_alibi_config(8), strict=False, opts={"tile_lists": False})
+    run(dev, torch.float32, 1, 4, 1, 130, 140, 128, scale=0.05, strict=False)
+
+
+def test_fp32_mfma_arbitrary_score_mod(dev):
+    """A score_mod outside the functor families (linearised into dense tables) on float32 inputs."""
+    def squash(score, b, h, q_idx, kv_idx):
+        return score * score * 0.1 + score
+    run(dev, torch.float32, 1, 2, 2, 96, 160, 64, score=squash, oscore=squash, mask=causal_mask, omask=o_causal_mask,
+        strict=False)
+
+
 # ---- faithful kernels, 16-bit, every functor ----
 SCORES = [
     ("identity", None, None),

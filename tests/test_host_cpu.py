@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     for name in decl:
         assert hasattr(L, name), name
-    assert L.flexattn_abi_version() == 3
+    assert L.flexattn_abi_version() == 4
     assert L.flexattn_last_error() is not None
 
 
@@ -61,7 +61,21 @@ def test_workspace_and_tile_queries_without_gpu():
     L.flexattn_preferred_tiles(_lib.FLEX_F16, 64, 64, 2048, 2048, 1, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (128, 128)
     L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
-    assert (qb.value, kvb.value) == (0, 0)
+    assert (qb.value, kvb.value) == (128, 64)      # the fp32 matrix-core kernels walk the same lists
+    L.flexattn_preferred_tiles(_lib.FLEX_F32, 256, 256, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (0, 0)         # generic kernels only: lists are ignored
+    # the kernel family is a pure function of the parameters
+    p = _lib.FlexAttnParams()
+    p.dtype, p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = _lib.FLEX_F32, 1, 2, 2, 256, 256, 64, 64
+    for name in ("q_stride", "k_stride", "v_stride", "o_stride"):
+        getattr(p, name)[:] = [2 * 256 * 64, 256 * 64, 64]
+    assert L.flexattn_kernel_family(p, 0) == 2 and L.flexattn_kernel_family(p, 1) == 2
+    p.flags = _lib.FLAG_STRICT
+    assert L.flexattn_kernel_family(p, 0) == 0
+    p.flags, p.dtype = 0, _lib.FLEX_BF16
+    assert L.flexattn_kernel_family(p, 0) == 1 and L.flexattn_kernel_family(p, 1) == 1
+    p.D = p.Dv = 256
+    assert L.flexattn_kernel_family(p, 0) == 0
     # argument validation happens before anything touches a device
     p = _lib.FlexAttnParams()
     assert L.flexattn_fwd(p, None, None, None, None, None, None, None) != 0
