@@ -39,9 +39,9 @@ selects numerics here:
                           whenever it applies (fp16/bf16, D = Dv in {64, 128},
                           at most 64 query rows per KV head, at least 512 keys)
     {"decode_splits": n}  force the split-KV decode kernel with n splits
-    {"pad_head_dim": bool}  inputs whose head sizes are not D = Dv in {64, 128} (but at most
-                          128) are zero-padded to the next of those so that the fused kernels serve
-                          them (default True)
+    {"pad_head_dim": bool}  inputs whose head sizes are not among those of the matrix-core kernels
+                          (D = Dv in {64, 128}, 16-bit inputs also {192, 256}) but no larger are
+                          zero-padded to the next of those (default True)
     {"tile_lists": bool}  False: call the library without tile lists, as a C-ABI caller without a
                           block mask would; every tile is then visited and the mask evaluated in
                           each (default True: lists are built from the mask)
@@ -446,18 +446,19 @@ def _as_kernel_layout(t: Array) -> Array:
 
 
 def _pad_head_dims(q: Array, k: Array, v: Array, kernel_options) -> Tuple[Array, Array, Array]:
-    """The matrix-core kernels (16-bit and float32) exist for D = Dv in {64, 128}.  Other head sizes up to 128
-    (and Dv < D) are zero-padded to the next of those: zero feature columns add nothing to Q.K^T, the
-    padded columns of O are dropped by the caller and the padded columns of the gradients are cut off by
-    autograd, so the result is the one of the original problem at matrix-core speed.  Opt out with
+    """The matrix-core kernels exist for D = Dv in {64, 128} and, for 16-bit inputs, {192, 256}.  Other head sizes
+    up to the largest of those (and Dv < D) are zero-padded to the next one: zero feature columns add nothing to
+    Q.K^T, the padded columns of O are dropped by the caller and the padded columns of the gradients are cut off
+    by autograd, so the result is the one of the original problem at matrix-core speed.  Opt out with
     kernel_options={"pad_head_dim": False}; the faithful and the generic kernels take any size as it is."""
     opts = kernel_options or {}
     D, Dv = q.shape[-1], v.shape[-1]
     if (q.dtype not in (torch.float16, torch.bfloat16, torch.float32) or opts.get("strict", False)
             or opts.get("backend", "auto") == "generic" or not opts.get("pad_head_dim", True)):
         return q, k, v
-    Dp = 64 if max(D, Dv) <= 64 else 128
-    if max(D, Dv) > 128 or (D == Dp and Dv == Dp):
+    sizes = (64, 128) if q.dtype == torch.float32 else (64, 128, 192, 256)
+    Dp = next((s for s in sizes if max(D, Dv) <= s), None)
+    if Dp is None or (D == Dp and Dv == Dp):
         return q, k, v
     pad = torch.nn.functional.pad
     return pad(q, (0, Dp - D)), pad(k, (0, Dp - D)), pad(v, (0, Dp - Dv))

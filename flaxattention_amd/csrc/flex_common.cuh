@@ -9,6 +9,7 @@ namespace flex {
 
 typedef _Float16 f16;
 typedef __bf16 bf16;
+typedef float f32;
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;

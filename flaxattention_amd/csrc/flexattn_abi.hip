@@ -30,10 +30,10 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
                        void* workspace, hipStream_t s);
 void* flex_decode_static_scratch(size_t* bytes);
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb);
-bool flex_f32_mfma_supported(const FlexAttnParams& p, int which);
-int flex_f32_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
-int flex_f32_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
-                      const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
+bool flex_simple_supported(const FlexAttnParams& p, int which);
+int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+int flex_simple_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
+                    const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
 
 static int validate(const FlexAttnParams* p, const char* who) {
   if (!p) { flex_set_error("%s: null params", who); return 1; }
@@ -102,7 +102,7 @@ static bool wants_fused(const FlexAttnParams* p) {
 
 extern "C" int flexattn_kernel_family(const FlexAttnParams* p, int32_t which) {
   if (!p || !wants_fused(p)) return FLEX_FAMILY_GENERIC;
-  if (flex_f32_mfma_supported(*p, which ? 1 : 0)) return FLEX_FAMILY_MFMA_F32;
+  if (flex_simple_supported(*p, which ? 1 : 0)) return p->dtype == FLEX_F32 ? FLEX_FAMILY_MFMA_F32 : FLEX_FAMILY_MFMA_16BIT;
   if (which ? flex_mfma_bwd_supported(*p) : flex_mfma_fwd_supported(*p)) return FLEX_FAMILY_MFMA_16BIT;
   return FLEX_FAMILY_GENERIC;
 }
@@ -121,10 +121,15 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o) { flex_set_error("flexattn_fwd: null tensor pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
-  // float32 inputs: the reference rounds nothing below fp32, so every numerics mode but FLEX_STRICT is the same
-  // computation and runs on the matrix cores
-  if (wants_fused(p) && flex_f32_mfma_supported(*p, 0)) {
-    if (int rc32 = flex_f32_mfma_fwd(*p, q, k, v, o, lse2, s)) return rc32;
+  // the simple matrix-core kernels: float32 inputs (the reference rounds nothing below fp32, so every numerics mode
+  // but FLEX_STRICT is the same computation) and the 16-bit head sizes above 128
+  if (wants_fused(p) && flex_simple_supported(*p, 0)) {
+    const FlexAttnParams ps = with_parity_resolved(p, true);
+    if ((ps.flags & FLEX_PARITY) && p->dtype != FLEX_F32 && !lse2) {
+      if (!workspace) { flex_set_error("flexattn_fwd: FLEX_PARITY needs lse2 or a workspace of flexattn_fwd_workspace_bytes()"); return 1; }
+      lse2 = (float*)workspace;
+    }
+    if (int rcs = flex_simple_fwd(ps, q, k, v, o, lse2, s)) return rcs;
     return check_launch("flexattn_fwd");
   }
   const bool fused = wants_fused(p) && flex_mfma_fwd_supported(*p);
@@ -159,8 +164,9 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
   if (!q || !k || !v || !o || !lse2 || !d_o || !dq || !dk || !dv || !workspace) { flex_set_error("flexattn_bwd: null pointer"); return 1; }
   hipStream_t s = (hipStream_t)stream;
   int rc;
-  if (wants_fused(p) && flex_f32_mfma_supported(*p, 1)) {
-    if (int rc32 = flex_f32_mfma_bwd(*p, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s)) return rc32;
+  if (wants_fused(p) && flex_simple_supported(*p, 1)) {
+    const FlexAttnParams ps = with_parity_resolved(p, true);
+    if (int rcs = flex_simple_bwd(ps, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s)) return rcs;
     return check_launch("flexattn_bwd");
   }
   const bool fused = wants_fused(p) && flex_mfma_bwd_supported(*p);

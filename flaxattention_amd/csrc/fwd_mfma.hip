@@ -24,9 +24,10 @@ bool flex_mfma_shape_ok(const FlexAttnParams& p) {
 }
 
 // which: 0 = forward and decode lists, 1 = backward lists
+bool flex_simple_shape(int dtype, int D, int Dv);
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
-  // the fp32 matrix-core kernels walk lists of the same granularity
-  const bool ok = (dtype == FLEX_F16 || dtype == FLEX_BF16 || dtype == FLEX_F32) && D == Dv && (D == 64 || D == 128);
+  // the simple matrix-core kernels (float32, 16-bit head sizes above 128) walk lists of the same granularity
+  const bool ok = ((dtype == FLEX_F16 || dtype == FLEX_BF16) && D == Dv && (D == 64 || D == 128)) || flex_simple_shape(dtype, D, Dv);
   *qb = !ok ? 0 : 128;
   *kvb = !ok ? 0 : (which == 0 ? kFwdBN : 128);
 }

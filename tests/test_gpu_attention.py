@@ -157,6 +157,9 @@ def test_kernel_family_query(dev):
         assert family(dev, torch.float16, 1, 4, 4, 256, 256, 64, causal_mask, bwd) == "mfma_16bit"
         assert family(dev, torch.bfloat16, 1, 4, 2, 100, 300, 128, None, bwd) == "mfma_16bit"
         assert family(dev, torch.bfloat16, 1, 4, 4, 256, 256, 64, None, bwd, {"backend": "generic"}) == "generic"
+        assert family(dev, torch.bfloat16, 1, 4, 4, 256, 256, 256, causal_mask, bwd) == "mfma_16bit"
+        assert family(dev, torch.float16, 1, 4, 2, 100, 300, 160, None, bwd) == "mfma_16bit"          # zero-padded to 192
+        assert family(dev, torch.float16, 1, 4, 4, 256, 256, 320, None, bwd) == "generic"
 
 
 SCORES_F32 = [
@@ -214,6 +217,39 @@ def test_fp32_mfma_arbitrary_score_mod(dev):
         return score * score * 0.1 + score
     run(dev, torch.float32, 1, 2, 2, 96, 160, 64, score=squash, oscore=squash, mask=causal_mask, omask=o_causal_mask,
         strict=False)
+
+
+# ---- 16-bit head sizes above 128 (192 and 256, others zero-padded to them) on the matrix cores ----
+WIDE = [
+    ("identity", None, None, causal_mask, o_causal_mask),
+    ("checker_kv", generate_checkerboard(2.0, 0.5, "kv"), o_checkerboard_kv, None, None),
+    ("alibi_cfg", generate_alibi_bias(4, sign=-1.0), o_alibi_config(4), causal_mask, o_causal_mask),
+    ("softcap_sink", generate_tanh_softcap(5.0), o_tanh_softcap(5.0), generate_attention_sink(50, 4), o_attention_sink(50, 4)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+@pytest.mark.parametrize("D", [192, 256])
+@pytest.mark.parametrize("name,score,oscore,mask,omask", WIDE, ids=[w[0] for w in WIDE])
+def test_wide_heads_default_numerics(dev, dtype, D, name, score, oscore, mask, omask):
+    """fp16 in its default ("fast") and bf16 in its default ("parity") numerics at the stated tolerance."""
+    print(f"case wide {name} {dtype} D{D}", flush=True)
+    run(dev, dtype, 2, 4, 4, 192, 256, D, score=score, oscore=oscore, mask=mask, omask=omask, strict=False)
+
+
+def test_wide_heads_other_modes(dev):
+    run(dev, torch.float16, 1, 2, 2, 160, 200, 256, mask=causal_mask, omask=o_causal_mask, strict=False,
+        opts={"numerics": "parity"})
+    run(dev, torch.bfloat16, 1, 2, 2, 160, 200, 256, mask=causal_mask, omask=o_causal_mask, strict=False,
+        opts={"numerics": "fast"})
+
+
+def test_wide_heads_gqa_ragged_padded_bitmap(dev):
+    def weird(b, h, q_idx, kv_idx):
+        return ((q_idx * 7 + kv_idx * 3 + h) % 11 < 6) & (q_idx % 5 != 0)
+    run(dev, torch.bfloat16, 2, 8, 2, 77, 203, 160, mask=causal_mask, omask=o_causal_mask,
+        score=generate_alibi_bias(8, -1.0), oscore=o_alibi_config(8), strict=False, opts={"tile_lists": False})
+    run(dev, torch.float16, 2, 3, 3, 100, 150, 224, Dv=200, mask=weird, omask=weird, strict=False)
 
 
 # ---- faithful kernels, 16-bit, every functor ----

@@ -62,6 +62,8 @@ def test_workspace_and_tile_queries_without_gpu():
     assert (qb.value, kvb.value) == (128, 128)
     L.flexattn_preferred_tiles(_lib.FLEX_F32, 64, 64, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (128, 64)      # the fp32 matrix-core kernels walk the same lists
+    L.flexattn_preferred_tiles(_lib.FLEX_BF16, 256, 256, 2048, 2048, 1, ctypes.byref(qb), ctypes.byref(kvb))
+    assert (qb.value, kvb.value) == (128, 128)
     L.flexattn_preferred_tiles(_lib.FLEX_F32, 256, 256, 2048, 2048, 0, ctypes.byref(qb), ctypes.byref(kvb))
     assert (qb.value, kvb.value) == (0, 0)         # generic kernels only: lists are ignored
     # the kernel family is a pure function of the parameters
@@ -75,6 +77,10 @@ def test_workspace_and_tile_queries_without_gpu():
     p.flags, p.dtype = 0, _lib.FLEX_BF16
     assert L.flexattn_kernel_family(p, 0) == 1 and L.flexattn_kernel_family(p, 1) == 1
     p.D = p.Dv = 256
+    assert L.flexattn_kernel_family(p, 0) == 1     # the 16-bit head sizes above 128 have matrix-core kernels too
+    p.D = p.Dv = 512
+    assert L.flexattn_kernel_family(p, 0) == 0
+    p.dtype, p.D, p.Dv = _lib.FLEX_F32, 256, 256
     assert L.flexattn_kernel_family(p, 0) == 0
     # argument validation happens before anything touches a device
     p = _lib.FlexAttnParams()
