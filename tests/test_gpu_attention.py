@@ -341,6 +341,24 @@ def test_bhln_false_layout(dev):
     close(out.transpose(1, 2), want, torch.float32, "O bhln=False")
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.bfloat16, 256), (torch.float16, 128)],
+                         ids=["f32_64", "bf16_256", "f16_128"])
+def test_bhln_false_layout_read_in_place(dev, dtype, D):
+    """[B,L,H,D] tensors reach every matrix-core kernel family through their strides, forward and backward."""
+    q, k, v = seeded_qkv(2, 4, 4, 96, 160, D, dtype)
+    d_o = torch.randn((2, 4, 96, D), generator=torch.Generator().manual_seed(3)).to(dtype)
+    want = ref_attention(q, k, v, None, o_causal_mask)
+    wq, wk, wv = ref_attention_bwd(q, k, v, d_o, None, o_causal_mask, strict=True)
+    qd, kd, vd = (t.transpose(1, 2).contiguous().to(dev).requires_grad_(True) for t in (q, k, v))   # [B,L,H,D]
+    out = fa.flax_attention_pallas(qd, kd, vd, mask_mod=causal_mask, bhln=False)
+    assert out.shape == (2, 96, 4, D)
+    close(out.transpose(1, 2), want, dtype, "O bhln=False")
+    out.backward(d_o.transpose(1, 2).contiguous().to(dev))
+    close(qd.grad.transpose(1, 2), wq, dtype, "dQ bhln=False")
+    close(kd.grad.transpose(1, 2), wk, dtype, "dK bhln=False")
+    close(vd.grad.transpose(1, 2), wv, dtype, "dV bhln=False")
+
+
 def test_untagged_score_mod_is_recognised(dev):
     def my_alibi(score, b, h, q_idx, kv_idx):
         return score + (q_idx - kv_idx) * torch.exp2(-((h + 1) * 8.0 / 8))
