@@ -175,10 +175,13 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   int t_cur = nt > 0 ? tile_at(0) : 0;
   int t_nxt = nt > 1 ? tile_at(1) : 0;
   // prologue: tile 0 into stage 0, tile 1 into registers
-  if (nt > 0) {
-    load_tile(t_cur * BN);
-    store_tile(0);
-  }
+  if (nt > 0) load_tile(t_cur * BN);
+  // Unconditional, and as an instruction the compiler's wait-count pass sees: the Q fragments (and tile 0) have
+  // arrived.  With the wait only inside the nt > 0 branch the pass carries "Q fragments may still be in flight" into
+  // the loop and makes the first products of every tile wait for all outstanding loads, i.e. for the prefetch of the
+  // tile after next that was issued half a tile earlier.
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+  if (nt > 0) store_tile(0);
   if (nt > 1) load_tile(t_nxt * BN);
   __syncthreads();
   for (int it = 0; it < nt; it++) {
