@@ -359,6 +359,43 @@ def test_bhln_false_layout_read_in_place(dev, dtype, D):
     close(vd.grad.transpose(1, 2), wv, dtype, "dV bhln=False")
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float16, 64), (torch.bfloat16, 64), (torch.float32, 64), (torch.bfloat16, 192)],
+                         ids=["f16_fast", "bf16_parity", "f32", "bf16_wide_parity"])
+def test_train_step_replays_from_a_captured_graph(dev, dtype, D):
+    """Forward and backward record into a HIP graph (no entry point synchronises, allocates outside the caller's
+    allocator or records a memset): every replay, with eager steps between the replays, gives the eager step's bits."""
+    print(f"case graph capture of a training step {dtype} D{D}", flush=True)
+    B, H, L = 2, 4, 384
+    g0 = torch.Generator(device="cpu").manual_seed(0)
+    mk = lambda: torch.randn(B, H, L, D, generator=g0, dtype=torch.float32).to(dtype).to(dev)
+    q, k, v = (mk().requires_grad_(True) for _ in range(3))
+    d_o = mk()
+    bm = fa.create_block_mask(causal_mask, 1, 1, L, L, device=dev)
+
+    def step():
+        out = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm)
+        return (out,) + torch.autograd.grad(out, (q, k, v), d_o)
+    side = torch.cuda.Stream()   # default priority; warm-up off the default stream as graph capture asks
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static = step()
+    for i in range(3):
+        with torch.no_grad():
+            for t in (q, k, v):
+                t.copy_(mk())
+        graph.replay()
+        eager = step()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("O", "dQ", "dK", "dV"), static, eager):
+            assert torch.equal(a, b), f"replay {i}: {name} differs from the eager step"
+
+
 def test_untagged_score_mod_is_recognised(dev):
     def my_alibi(score, b, h, q_idx, kv_idx):
         return score + (q_idx - kv_idx) * torch.exp2(-((h + 1) * 8.0 / 8))
