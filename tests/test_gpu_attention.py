@@ -704,6 +704,24 @@ def test_fused_seeded_sweep(dev, seed):
             mask=c["mask"], omask=c["omask"], strict=False, scale_maxabs=True)
 
 
+@pytest.mark.parametrize("seed", range(100, 116))
+def test_simple_kernels_seeded_sweep(dev, seed):
+    """The same sweep over the shapes of the simple matrix-core kernels: float32 (D 32 .. 128) and 16-bit head sizes
+    above 128 (160 is zero-padded to 192)."""
+    import random
+    c = _sweep_case(seed)
+    rnd = random.Random(seed)
+    if rnd.random() < 0.5:
+        c["dtype"], c["D"] = torch.float32, rnd.choice([32, 64, 96, 128])
+    else:
+        c["D"] = rnd.choice([160, 192, 256])
+    print(f"sweep {seed}: {c['dtype']} B{c['B']} Hq{c['Hq']} Hkv{c['Hkv']} Lq{c['Lq']} Lkv{c['Lkv']} D{c['D']} "
+          f"score {c['name']} mask {getattr(c['mask'], '__name__', c['mask'])} block_mask {c['use_block_mask']}", flush=True)
+    pallas = c["mask"] is not None and not c["use_block_mask"]
+    run(dev, c["dtype"], c["B"], c["Hq"], c["Hkv"], c["Lq"], c["Lkv"], c["D"], score=c["score"], oscore=c["oscore"],
+        mask=c["mask"], omask=c["omask"], strict=False, pallas=pallas, scale_maxabs=True)
+
+
 # ---- score_mods that add a captured bias: a dense additive table read by the fused kernels ----
 def test_fused_additive_bias_table(dev):
     g = torch.Generator().manual_seed(11)
