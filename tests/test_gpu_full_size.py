@@ -157,3 +157,33 @@ def test_config5_full_size(dev, Lq):
         print(f"  (b{b},h{h}): O max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
         assert a <= 2e-2 and r <= 1e-3
         assert max_abs(lse[b:b + 1, h:h + 1].cpu(), want_lse) <= 2e-2
+
+
+@pytest.mark.parametrize("dtype,D,B,H,L", [(torch.float16, 128, 33, 32, 16384), (torch.float32, 128, 33, 32, 16384),
+                                           (torch.bfloat16, 256, 17, 32, 16384)],
+                         ids=["f16_d128_tuned", "f32_d128_simple", "bf16_d256_simple"])
+def test_tensors_beyond_2_31_elements(dev, dtype, D, B, H, L):
+    """Q, K, V, O and the gradients hold more than 2^31 elements each (and more than 2^32 bytes), so every row address
+    of the last batch element lies beyond what 32 bits reach.  The (batch, head) pairs of a call are independent
+    and their tile schedules identical, so the last pair's slice of the big call must equal, bit for bit, a call on
+    that slice alone (whose addresses are small): forward, lse, dQ, dK, dV under a causal block mask."""
+    assert B * H * L * D > 2 ** 31
+    g = torch.Generator(device=dev).manual_seed(5)
+    mk = lambda: torch.randn((B, H, L, D), generator=g, dtype=torch.float32 if dtype == torch.float32 else torch.float16,
+                             device=dev).to(dtype)
+    q, k, v = (mk().requires_grad_(True) for _ in range(3))
+    d_o = mk()
+    bm = fa.create_block_mask(causal_mask, 1, 1, L, L, device=dev)
+    score = generate_alibi_bias(H, -1.0)
+    out, lse = fa.flax_attention(q, k, v, score_mod=score, block_mask=bm, return_lse=True)
+    gq, gk, gv = torch.autograd.grad(out, (q, k, v), d_o)
+    b, h = B - 1, H - 1
+    qs, ks, vs = (t[b:b + 1, h:h + 1].detach().clone().requires_grad_(True) for t in (q, k, v))
+    # head H-1 of H has the ALiBi slope 2^-8, and so has head 0 of 1
+    shifted = generate_alibi_bias(1, -1.0)
+    out1, lse1 = fa.flax_attention(qs, ks, vs, score_mod=shifted, block_mask=bm, return_lse=True)
+    gq1, gk1, gv1 = torch.autograd.grad(out1, (qs, ks, vs), d_o[b:b + 1, h:h + 1].clone())
+    torch.cuda.synchronize()
+    for name, big, small in (("O", out, out1), ("lse", lse, lse1), ("dQ", gq, gq1), ("dK", gk, gk1), ("dV", gv, gv1)):
+        sl = big[b:b + 1, h:h + 1]
+        assert torch.equal(sl, small), f"{name}: slice of the big call differs from the call on the slice"
