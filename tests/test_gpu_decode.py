@@ -186,3 +186,25 @@ def test_calls_replay_from_a_captured_graph(dev, Lq):
         eager, eager_lse = call(q_new)
         torch.cuda.synchronize()
         assert torch.equal(out_static, eager) and torch.equal(lse_static, eager_lse), f"replay {i} differs from the eager call"
+
+
+@pytest.mark.parametrize("Lq", [1, 64])
+def test_decode_kv_cache_beyond_2_31_elements(dev, Lq):
+    """A KV cache of more than 2^31 elements per tensor (more than 2^32 bytes): the rows of its last (batch, head) pair
+    lie beyond what 32 bits address.  The pairs of a call are independent, so the last pair's output must equal,
+    bit for bit, a decode call on that pair's slice of the cache alone."""
+    B, H, Lkv, D = 33, 16, 65536, 64
+    assert B * H * Lkv * D > 2 ** 31
+    g = torch.Generator(device=dev).manual_seed(9)
+    mk = lambda *s: torch.randn(s, generator=g, dtype=torch.float16, device=dev)
+    K, V, q = mk(B, H, Lkv, D), mk(B, H, Lkv, D), mk(B, H, Lq, D)
+    bm = fa.create_block_mask(offset_causal_mask(Lkv - Lq), 1, 1, Lq, Lkv, device=dev)
+    opts = {"decode_splits": 4}
+    out, lse = fa.flax_attention(q, K, V, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True,
+                                 kernel_options=opts)
+    b, h = B - 1, H - 1
+    # head H-1 of H has the ALiBi slope 2^-8, and so has head 0 of 1
+    out1, lse1 = fa.flax_attention(q[b:b + 1, h:h + 1].clone(), K[b:b + 1, h:h + 1].clone(), V[b:b + 1, h:h + 1].clone(),
+                                   score_mod=generate_alibi_bias(1, -1.0), block_mask=bm, return_lse=True, kernel_options=opts)
+    torch.cuda.synchronize()
+    assert torch.equal(out[b:b + 1, h:h + 1], out1) and torch.equal(lse[b:b + 1, h:h + 1], lse1)
