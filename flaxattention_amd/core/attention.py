@@ -542,8 +542,9 @@ def kernel_family(query: Array, key: Array, value: Array, score_mod: Optional[_s
                   block_mask: Optional[BlockMask] = None, scale: Optional[float] = None,
                   kernel_options: Optional[Dict[str, Any]] = None, backward: bool = False) -> str:
     """Which kernels flax_attention runs for these inputs: "generic" (vector ALU), "mfma_16bit" or "mfma_f32"
-    (matrix cores).  Asks the library (flexattn_kernel_family) with the parameters the call itself would pass;
-    nothing is computed.  No counterpart in the reference, which has one dense path (core/attention.py:14-106)."""
+    (matrix cores).  Asks the library (flexattn_kernel_family) with the parameters the call itself would pass: the
+    score_mod and the mask are lowered and the mask's tile lists built as the call would, no attention is computed.
+    No counterpart in the reference, which has one dense path (core/attention.py:14-106)."""
     _require_device(query, key, value)
     if score_mod is None:
         score_mod = _identity
