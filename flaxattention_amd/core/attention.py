@@ -560,7 +560,7 @@ def kernel_family(query: Array, key: Array, value: Array, score_mod: Optional[_s
         opts = dict(kernel_options or {})
         opts["tile_lists"] = opts.get("tile_lists", True)
         plan = _make_plan(q, k, v, _identity, block_mask, None, scale, opts)
-        plan.score = ScoreMod(_lib.SCORE_AFFINE, mul=torch.ones(1, device=q.device), add=None)
+        plan.score = ScoreMod(_lib.SCORE_AFFINE, mul=torch.ones((1, 1, 1, 1), device=q.device), add=None)
     o_like = torch.empty((q.shape[0], q.shape[1], q.shape[2], v.shape[3]), dtype=q.dtype, device="meta")
     p = plan.params(q, k, v, o_like)
     return _FAMILIES[_lib.lib().flexattn_kernel_family(_lib.C.byref(p), 1 if backward else 0)]

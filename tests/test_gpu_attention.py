@@ -160,6 +160,9 @@ def test_kernel_family_query(dev):
         assert family(dev, torch.bfloat16, 1, 4, 4, 256, 256, 256, causal_mask, bwd) == "mfma_16bit"
         assert family(dev, torch.float16, 1, 4, 2, 100, 300, 160, None, bwd) == "mfma_16bit"          # zero-padded to 192
         assert family(dev, torch.float16, 1, 4, 4, 256, 256, 320, None, bwd) == "generic"
+    # a score_mod outside the functor families is linearised into dense tables, which the matrix-core kernels read
+    q = torch.zeros((1, 2, 64, 64), dtype=torch.float16, device=dev)
+    assert fa.kernel_family(q, q, q, score_mod=lambda s, b, h, qi, ki: s * s) == "mfma_16bit"
 
 
 SCORES_F32 = [
