@@ -725,6 +725,17 @@ def test_simple_kernels_seeded_sweep(dev, seed):
         mask=c["mask"], omask=c["omask"], strict=False, pallas=pallas, scale_maxabs=True)
 
 
+@pytest.mark.parametrize("dtype,D", [(torch.float32, 64), (torch.float32, 128), (torch.bfloat16, 192), (torch.float16, 256),
+                                     (torch.float16, 64), (torch.bfloat16, 128)],
+                         ids=["f32_64", "f32_128", "bf16_192", "f16_256", "f16_64", "bf16_128"])
+def test_tiny_and_odd_shapes_on_every_family(dev, dtype, D):
+    """Sequence lengths far below a tile, one key, one row, odd head counts: every matrix-core kernel family."""
+    for B, Hq, Hkv, Lq, Lkv, mask, omask in ((1, 1, 1, 1, 1, None, None), (3, 5, 5, 5, 7, causal_mask, o_causal_mask),
+                                             (1, 6, 3, 33, 31, None, None), (2, 7, 1, 2, 129, causal_mask, o_causal_mask)):
+        print(f"case tiny {dtype} D{D} B{B} Hq{Hq} Hkv{Hkv} Lq{Lq} Lkv{Lkv}", flush=True)
+        run(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, mask=mask, omask=omask, strict=False, scale_maxabs=True)
+
+
 # ---- score_mods that add a captured bias: a dense additive table read by the fused kernels ----
 def test_fused_additive_bias_table(dev):
     g = torch.Generator().manual_seed(11)
