@@ -41,8 +41,13 @@ constexpr int kListBN = 128; // key granularity of the backward tile lists = key
 //   kBwdHiLo     dQ of the "unrounded" numerics: reads that delta; dP stays in fp32 and dS goes into the product
 //                as a high and a low part (two matrix instructions per fragment); launched with ROUND_S = false
 enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2, kBwdDeltaRaw = 3, kBwdHiLo = 4 };
+// Registers: two waves per SIMD (256 registers each) everywhere but the fast-numerics kernel at D = 128, which then
+// spills 31 - 59 registers and reloads them inside the tile loop (every reload is a vector memory load, and a wait for
+// one is a wait for the tile fetch in flight as well); with one wave per SIMD and no spill it is 10 - 15 % faster
+// ([4,16,4096,128] bf16: 1213 -> 1031 us dense, 603 -> 544 us causal).  The row sweep does not spill; the parity kernel
+// (19 - 52 registers spilled) loses 22 % with one wave per SIMD and the high/low kernel gains nothing, so they keep two.
 template <typename T, int D, int KIND, bool ROUND_S, bool MASKED, int MODE = kBwdFast>
-__global__ __launch_bounds__(256, 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, (D == 128 && MODE == kBwdFast) ? 1 : 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
                                                       const T* __restrict__ d_o, T* __restrict__ dq,
