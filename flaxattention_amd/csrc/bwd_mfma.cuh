@@ -359,12 +359,12 @@ extern __shared__ __align__(16) unsigned char bwd_smem[];
 // four 32-row query blocks of a tile in turn, so a Q / dO tile fetched from L2 serves 128 keys
 // and nothing has to be summed across waves.  With D = 64 two such workgroups share a
 // compute unit (two waves per SIMD); being independent they drift out of phase, so one's
-// matrix work overlaps the other's vector work and barrier waits.
+// matrix work overlaps the other's vector work and barrier waits.  With D = 128 a wave holds
+// 410 - 430 registers (128 of them dK / dV accumulators), so one workgroup has the compute unit.
 template <int D> struct DkvShape {
   static constexpr int kWaves = kListBN / 32;
   static constexpr int kThreads = kWaves * 64;
   static constexpr int kQBlocks = kBM / 32;        // 32-row query blocks per wave and tile
-  static constexpr int kStages = D == 64 ? 2 : 1;  // LDS stages of the query-side tiles
 };
 
 // BITS: the mask is a bitmap.  Band masks get an instantiation of their own, without the bitmap code: with it in the
@@ -381,18 +381,14 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
                                                                const T* __restrict__ d_o, T* __restrict__ dk,
                                                                T* __restrict__ dv) {
   typedef typename Frag<T>::vec8 vec8;
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int BM = kBM, BN = kListBN;
-  constexpr int kDkvThreads = DkvShape<D>::kThreads, QBW = DkvShape<D>::kQBlocks;
-  // D = 64: the Q and dO tiles land in LDS straight from global memory (unpadded rows, chunk c of row r at
-  // position c ^ lds_swz(r): conflict-free for the row-fragment and the transposing reads); D = 128 stages them
-  // through registers into padded rows
-  constexpr bool DIRECT = D == 64;
-  constexpr int DS = D / 16, DB = D / 32, ROWE = DIRECT ? D : D + 8, CPR = D / 8, NLD = BM * CPR / kDkvThreads;
-  // LDS stages of (Q tile, dO tile, lse, -delta).  D = 64 keeps two, so that one workgroup
-  // barrier per tile suffices; with D = 128 a second stage would cost the second workgroup
-  // of the compute unit, so one stage is refilled between two barriers.
-  constexpr int NSTG = DkvShape<D>::kStages;
+  constexpr int QBW = DkvShape<D>::kQBlocks;
+  // The Q and dO tiles land in LDS straight from global memory (unpadded rows, chunk c of row r at position
+  // c ^ lds_swz(r): conflict-free for the row-fragment and the transposing reads), one tile ahead of the one being
+  // read, into two stages of (Q tile, dO tile, lse, -delta): one workgroup barrier per tile.  (At D = 128 this replaced
+  // one stage filled through registers between two barriers: [4,16,4096,128] bf16 1425 -> 1345 us dense, 828 -> 733 us
+  // causal in the parity numerics.)
+  constexpr int DS = D / 16, DB = D / 32, ROWE = D, CPR = D / 8;
   constexpr int kStageBytes = 2 * BM * ROWE * (int)sizeof(T) + 2 * BM * (int)sizeof(float);
   auto stage_q = [&](int st) { return reinterpret_cast<T*>(bwd_smem + st * kStageBytes); };
 
@@ -423,7 +419,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
     for (int r = 0; r < 16; r++) { dkacc[db][r] = 0.f; dvacc[db][r] = 0.f; }
   // element offsets inside a 32-row block of a tile: row fragments (row i32, chunk 2s + g) and transposing
   // reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
-  const int kz = DIRECT ? (g ^ lds_swz<D>(i32)) : g;
+  const int kz = g ^ lds_swz<D>(i32);
   int toff[2][DB];
   {
     const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
@@ -432,7 +428,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
 #pragma unroll
       for (int db = 0; db < DB; db++) {
         const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
-        const int pos = DIRECT ? (chunk ^ lds_swz<D>(rl + 8 * e)) : chunk;
+        const int pos = chunk ^ lds_swz<D>(rl + 8 * e);
         toff[e][db] = (rl + 8 * e) * ROWE + pos * 8 + 4 * (i16 & 1);
       }
   }
@@ -467,19 +463,19 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       if (!full_idx) return it;
       return uniform_ld(it < n_full ? full_idx + it : part_idx + (it - n_full));
     };
-    u32x4 qreg[DIRECT ? 1 : NLD], oreg[DIRECT ? 1 : NLD];
-    float lreg = INFINITY, dreg = 0.f;
-    // direct fetch: wave w fills rows [32w, 32w + 32) of the Q and the dO tile, 8 rows per instruction; the lane
+    float lreg = INFINITY, dreg = 0.f;  // lse and delta of the tile after next, one row per thread
+    // tile fetch: wave w fills rows [32w, 32w + 32) of the Q and the dO tile, 64 / CPR rows per instruction; the lane
     // that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
     auto issue_tile = [&](int st, int q0) {
       T* Qw = stage_q(st);
       T* Ow = Qw + BM * ROWE;
+      constexpr int RPI = 64 / CPR, NI = 32 / RPI;  // rows per fetch instruction, instructions per wave and tensor
       const int lim = p.Lq - 1 - q0;  // rows past the end: clamped (finite filler; their lse is +inf, so P = 0)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int r0 = 32 * w + 8 * j;
-        const int chunk = (lane & 7) ^ lds_swz<D>(8 * j + (lane >> 3));  // the wave's first row is a multiple of 16
-        const int row = min(r0 + (lane >> 3), lim);
+      for (int j = 0; j < NI; j++) {
+        const int r0 = 32 * w + RPI * j;
+        const int chunk = (lane % CPR) ^ lds_swz<D>(RPI * j + lane / CPR);  // the wave's first row is a multiple of 16
+        const int row = min(r0 + lane / CPR, lim);
         const T* qg = qbase + (int64_t)(q0 + row) * p.q_stride[2] + chunk * 8;
         const T* og = dobase + (int64_t)(q0 + row) * D + chunk * 8;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)qg,
@@ -489,14 +485,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       }
     };
     auto load_tile = [&](int q0) {
-      if constexpr (!DIRECT) {
-#pragma unroll
-        for (int j = 0; j < NLD; j++) {
-          const int c = tid + kDkvThreads * j, r = min(c / CPR, p.Lq - 1 - q0), cc = c % CPR;  // clamped: finite filler
-          qreg[j] = *reinterpret_cast<const u32x4*>(qbase + (int64_t)(q0 + r) * p.q_stride[2] + cc * 8);
-          oreg[j] = *reinterpret_cast<const u32x4*>(dobase + (int64_t)(q0 + r) * D + cc * 8);
-        }
-      }
       lreg = INFINITY;
       dreg = 0.f;
       if (tid < BM && q0 + tid < p.Lq) {
@@ -511,14 +499,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       T* Qw = stage_q(st);
       T* Ow = Qw + BM * ROWE;
       float* lw = reinterpret_cast<float*>(Ow + BM * ROWE);
-      if constexpr (!DIRECT) {
-#pragma unroll
-        for (int j = 0; j < NLD; j++) {
-          const int c = tid + kDkvThreads * j, r = c / CPR, cc = c % CPR;
-          *reinterpret_cast<u32x4*>(Qw + r * ROWE + cc * 8) = qreg[j];
-          *reinterpret_cast<u32x4*>(Ow + r * ROWE + cc * 8) = oreg[j];
-        }
-      }
       if (tid < BM) {
         lw[tid] = lreg;        // rows past Lq carry lse = +inf: P = 0, whatever the clamped loads hold
         lw[BM + tid] = -dreg;  // the dP accumulator starts from -delta
@@ -526,43 +506,31 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
     };
     __syncthreads();  // the stages may still be in use by the previous head of the group
     if (nt > 0) {
-      if constexpr (DIRECT) issue_tile(0, t_cur * BM);
+      issue_tile(0, t_cur * BM);
       load_tile(t_cur * BM);
+      store_tile(0);
     }
-    if (NSTG == 2) {
-      if (nt > 0) store_tile(0);
-      if (nt > 1) load_tile(t_nxt * BM);
-      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-    }
+    if (nt > 1) load_tile(t_nxt * BM);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     for (int it = 0; it < nt; it++) {
       const int q0 = t_cur * BM;
       const bool masked = (it >= n_full) || (q0 + BM > p.Lq) || (kt * BN + BN > p.Lkv);
-      const int st = NSTG == 2 ? (it & 1) : 0;
-      const T* Qs = stage_q(st);
+      const T* Qs = stage_q(it & 1);
       const T* Os = Qs + BM * ROWE;
       const float* lse_s = reinterpret_cast<const float*>(Os + BM * ROWE);
       const float* del_s = lse_s + BM;
-      if (NSTG == 2) {
-        if (it + 1 < nt) {
-          // the other stage was last read before the previous barrier: refill it (D = 64: the
-          // tile itself is fetched straight into it now and awaited at the end of this tile; lse
-          // and delta, like whole tiles at D = 128, were prefetched into registers), then start
-          // fetching the one after
-          if constexpr (DIRECT) issue_tile((it + 1) & 1, t_nxt * BM);
-          store_tile((it + 1) & 1);
-          t_cur = t_nxt;
-          if (it + 2 < nt) {
-            t_nxt = tile_at(it + 2);
-            load_tile(t_nxt * BM);
-          }
-        }
-      } else {
-        store_tile(0);  // the barrier that closed the previous tile freed the stage
-        __syncthreads();
-        if (it + 1 < nt) load_tile(t_nxt * BM);
+      if (it + 1 < nt) {
+        // the other stage was last read before the previous barrier: refill it (the tile itself is fetched
+        // straight into it now and awaited at the end of this tile; lse and delta were prefetched into
+        // registers), then start fetching the lse and delta of the one after
+        issue_tile((it + 1) & 1, t_nxt * BM);
+        store_tile((it + 1) & 1);
         t_cur = t_nxt;
-        if (it + 2 < nt) t_nxt = tile_at(it + 2);
+        if (it + 2 < nt) {
+          t_nxt = tile_at(it + 2);
+          load_tile(t_nxt * BM);
+        }
       }
 
 #pragma unroll
@@ -602,19 +570,17 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
           dpacc = Frag<T>::mfma(*reinterpret_cast<const vec8*>(op + (((2 * s) ^ kz) * 8)), vf[s], dpacc);
         }
       }
-      // D = 64 has the registers to fetch the transposed dO and Q fragments of the closing products now, under the
-      // softmax arithmetic, instead of right before their use (1.7 % of the kernel's time)
+      // the transposed dO and Q fragments of the closing products are fetched now, under the softmax arithmetic,
+      // instead of right before their use (D = 64: 1.7 % of the kernel's time)
       vec8 a_do[2][DB], a_q[2][DB];
-      if constexpr (DIRECT) {
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
+      for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-          for (int db = 0; db < DB; db++) {
-            const int base = (qrow_w + 16 * tt) * ROWE;
-            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
-            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
-          }
-      }
+        for (int db = 0; db < DB; db++) {
+          const int base = (qrow_w + 16 * tt) * ROWE;
+          a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
+          a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
+        }
       // x = log2(e) * score_mod(scale * s) - lse_q  (P = 2^x), dp <- dP - delta_q
       float16_t gacc;
       if constexpr (KIND == kScoreCheckerboardKv) key_grad = sm.key_grad;
@@ -680,11 +646,6 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
       for (int tt = 0; tt < 2; tt++) {
 #pragma unroll
         for (int db = 0; db < DB; db++) {
-          const int base = (qrow_w + 16 * tt) * ROWE;
-          if constexpr (!DIRECT) {
-            a_do[tt][db] = join8<vec8>(lds_read_tr(Os + base + toff[0][db]), lds_read_tr(Os + base + toff[1][db]));
-            a_q[tt][db] = join8<vec8>(lds_read_tr(Qs + base + toff[0][db]), lds_read_tr(Qs + base + toff[1][db]));
-          }
           dvacc[db] = Frag<T>::mfma(a_do[tt][db], pf[tt], dvacc[db]);
           dkacc[db] = Frag<T>::mfma(a_q[tt][db], dsf[tt], dkacc[db]);
           if constexpr (HILO) {
@@ -694,7 +655,7 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
         }
       }
       }  // query blocks of this wave
-      if constexpr (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the next tile has landed
       __syncthreads();
     }
   }
@@ -720,8 +681,9 @@ __global__ __launch_bounds__(DkvShape<D>::kThreads, D == 64 ? 2 : 1) void bwd_dk
   }
 }
 
+// two stages of (Q tile, dO tile, lse, -delta)
 template <int D, typename T> constexpr size_t dkv_smem() {
-  return DkvShape<D>::kStages * ((size_t)2 * kBM * (D == 64 ? D : D + 8) * sizeof(T) + 2 * kBM * sizeof(float));
+  return 2 * ((size_t)2 * kBM * D * sizeof(T) + 2 * kBM * sizeof(float));
 }
 
 // everything a backward launch needs besides the template choice
