@@ -41,6 +41,8 @@ constexpr int kListBN = 128; // key granularity of the backward tile lists = key
 //   kBwdHiLo     dQ of the "unrounded" numerics: reads that delta; dP stays in fp32 and dS goes into the product
 //                as a high and a low part (two matrix instructions per fragment); launched with ROUND_S = false
 enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2, kBwdDeltaRaw = 3, kBwdHiLo = 4 };
+// keys the dQ kernel stages per step (the kernel and the launcher that picks its mask-free instantiation agree on it)
+template <int D, int MODE> constexpr int dq_tile_keys() { return (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2; }
 // Registers: two waves per SIMD (256 registers each) everywhere but the fast-numerics kernel at D = 128, which then
 // spills 31 - 59 registers and reloads them inside the tile loop (every reload is a vector memory load, and a wait for
 // one is a wait for the tile fetch in flight as well); with one wave per SIMD and no spill it is 10 - 15 % faster
@@ -56,7 +58,7 @@ __global__ __launch_bounds__(256, (D == 128 && MODE == kBwdFast) ? 1 : 2) void b
   // keys staged per step: 128 at D = 64, 64 at D = 128, so that two stages of K and V are 64 KB
   // either way and two workgroups (two waves per SIMD) share a compute unit; the fast-numerics kernel at
   // D = 128 runs one wave per SIMD (see above), has the 128 KB for 128-key tiles and is 3 - 6 % faster with them
-  constexpr int BM = kBM, BN = (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2;
+  constexpr int BM = kBM, BN = dq_tile_keys<D, MODE>();
   constexpr int DS = D / 16, DB = D / 32, CPR = D / 8;
   constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
   constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor
@@ -724,7 +726,7 @@ static void launch_dq_as(const FlexAttnParams& p, const BwdArgs& a) {
 
 template <typename T, int D, int KIND, bool RS>
 static void launch_dq(const FlexAttnParams& p, const BwdArgs& a) {
-  constexpr int BN = D == 64 ? kBN : kBN / 2;   // the kernel's key tile
+  constexpr int BN = dq_tile_keys<D, kBwdFast>();   // the kernel's key tile
   if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0) launch_dq_as<T, D, KIND, RS, false, kBwdFast>(p, a);
   else launch_dq_as<T, D, KIND, RS, true, kBwdFast>(p, a);
 }
