@@ -201,19 +201,25 @@ def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
         return 0
     B, Hq, Lq, D = q.shape
     G = Hq // k.shape[1]
-    ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128)
+    ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128, 256)
           and score.kind != _lib.SCORE_AFFINE
           and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC | _lib.FLAG_UNROUNDED)))
     if want is True:
         return -1   # the library reports what does not fit
     if not ok:
         return 0
-    if G * Lq <= 64:
+    cols = _decode_columns(D)
+    if G * Lq <= cols:
         return -1 if k.shape[2] >= 512 else 0
-    # 65..256 rows against a long KV cache: a few decode passes over the cache beat a forward grid
-    # that would leave most compute units without a workgroup (one per 128 query rows and head)
+    # up to four calls' worth of rows against a long KV cache: a few decode passes over the cache beat a forward
+    # grid that would leave most compute units without a workgroup (one per 128 query rows and head)
     few_workgroups = B * Hq * ((Lq + 127) // 128) < 256
-    return -1 if (G == 1 and Lq <= 256 and k.shape[2] >= 4096 and few_workgroups) else 0
+    return -1 if (G == 1 and Lq <= 4 * cols and k.shape[2] >= 4096 and few_workgroups) else 0
+
+
+def _decode_columns(D: int) -> int:
+    """Query columns (rows x heads per KV head) one decode call takes."""
+    return 32 if D > 128 else 64
 
 
 _holders: dict = {}
@@ -246,12 +252,12 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     with torch.cuda.device(q.device):
         if plan.decode_splits != 0:
             splits = max(plan.decode_splits, 0)   # 0 asks the library for its default
-            rows = max(64 // (plan.Hq // plan.Hkv), 1)   # query rows one decode call takes
+            rows = max(_decode_columns(plan.D) // (plan.Hq // plan.Hkv), 1)   # query rows one decode call takes
             if plan.Lq <= rows:
                 chunks = [(0, plan.Lq, q, o, lse2, p)]
             else:
-                # a longer query goes through the decode kernel 64 rows at a time (rows is 64 here:
-                # chunking is only chosen without GQA packing), each call seeing its row offset
+                # a longer query goes through the decode kernel 64 (D = 256: 32) rows at a time (chunking is
+                # only chosen without GQA packing), each call seeing its row offset
                 chunks = []
                 for s0 in range(0, plan.Lq, rows):
                     s1 = min(s0 + rows, plan.Lq)

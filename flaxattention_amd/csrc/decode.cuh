@@ -16,11 +16,14 @@ constexpr int kStep = 32;  // KV rows per wave step
 //                kernel sums them)
 enum { kDecOnePass = 0, kDecLse = 1, kDecNorm = 2 };
 template <typename T, int D, int KIND, bool ROUND_S, int NB, int PASS = kDecOnePass>
-__global__ __launch_bounds__(256, NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D == 256 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits, const float* __restrict__ lse_in) {
   typedef typename Frag<T>::vec8 vec8;
+  // D = 256 serves one column block: the two V strips of the four waves are 128 KB of the 160 KB of LDS, which leaves
+  // no room for a second block's Q fragments, and its registers (64 for Q, 64 for K, 128 for O) no room to keep them
+  static_assert(D == 64 || D == 128 || (D == 256 && NB == 1), "decode_split_kernel: head size / column blocks");
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8;
   constexpr int RPI = 64 / CPR;        // V rows one wave-wide fetch instruction fills
   constexpr int NVI = kStep / RPI;     // fetch instructions per step
@@ -437,12 +440,13 @@ template <typename T, int D, int KIND, bool RS, int PASS>
 static void launch_nb(const FlexAttnParams& p, const DecodeArgs& a) {
   dim3 grid(a.splits, p.Hkv, p.B);
   const int ncols = (p.Hq / p.Hkv) * p.Lq;
-  if (ncols <= 32)
+  if (ncols <= 32 || D == 256) {  // the caller has checked that D = 256 comes with at most 32 columns
     hipLaunchKernelGGL((decode_split_kernel<T, D, KIND, RS, 1, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
                        (const T*)a.v, a.o_part, a.ml_part, a.splits, a.lse_pass);
-  else
+  } else if constexpr (D != 256) {
     hipLaunchKernelGGL((decode_split_kernel<T, D, KIND, RS, 2, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
                        (const T*)a.v, a.o_part, a.ml_part, a.splits, a.lse_pass);
+  }
 }
 
 template <typename T, int D>

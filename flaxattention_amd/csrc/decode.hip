@@ -1,4 +1,4 @@
-// Split-KV decode for gfx950: short queries (G * Lq <= 64 columns) against a
+// Split-KV decode for gfx950: short queries (G * Lq <= 64 columns; 32 at D = 256) against a
 // long KV cache, bound by HBM bandwidth.
 //
 // Serves the decode shapes of examples/benchmark_decoding.py:29-33 (the
@@ -31,12 +31,24 @@ int flex_decode_f16_64(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_f16_128(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_64(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_128(const FlexAttnParams& p, const DecodeArgs& a);
+int flex_decode_f16_256(const FlexAttnParams& p, const DecodeArgs& a);
+int flex_decode_bf16_256(const FlexAttnParams& p, const DecodeArgs& a);
 void flex_set_error(const char* fmt, ...);
 bool flex_mfma_shape_ok(const FlexAttnParams& p);
 
+// 16-bit inputs, D = Dv in {64, 128} with up to 64 query columns (rows x heads per KV head) or D = Dv = 256 with up to 32
 bool flex_decode_supported(const FlexAttnParams& p) {
-  if (!flex_mfma_shape_ok(p) || p.score.kind == FLEX_SCORE_AFFINE) return false;
-  return (int64_t)(p.Hq / p.Hkv) * p.Lq <= 64 && p.Hkv <= 65535 && p.B <= 65535;
+  if (p.score.kind == FLEX_SCORE_AFFINE) return false;
+  int max_cols = 64;
+  if (p.D == 256 && p.Dv == 256) {
+    FlexAttnParams as128 = p;  // dtype, stride and grid checks are those of the narrower heads
+    as128.D = as128.Dv = 128;
+    if (!flex_mfma_shape_ok(as128)) return false;
+    max_cols = 32;
+  } else if (!flex_mfma_shape_ok(p)) {
+    return false;
+  }
+  return (int64_t)(p.Hq / p.Hkv) * p.Lq <= max_cols && p.Hkv <= 65535 && p.B <= 65535;
 }
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
@@ -100,8 +112,8 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
   float* lse_ws = ml_part + rows * splits * 2;
   const DecodeArgs a = {q, k, v, o, lse2, lse2 ? lse2 : lse_ws, o_part, ml_part, splits, s};
   int rc;
-  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_decode_f16_64(p, a) : flex_decode_f16_128(p, a);
-  else rc = p.D == 64 ? flex_decode_bf16_64(p, a) : flex_decode_bf16_128(p, a);
+  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_decode_f16_64(p, a) : p.D == 128 ? flex_decode_f16_128(p, a) : flex_decode_f16_256(p, a);
+  else rc = p.D == 64 ? flex_decode_bf16_64(p, a) : p.D == 128 ? flex_decode_bf16_128(p, a) : flex_decode_bf16_256(p, a);
   if (rc) flex_set_error("decode: unsupported score_mod kind %d", p.score.kind);
   return rc;
 }

@@ -155,8 +155,8 @@ typedef struct FlexAttnParams {
   FlexTileLists tiles_bwd; /* lists for flexattn_bwd (its kernels tile differently) */
   /* flexattn_decode only (0 elsewhere): the query tensor passed in is rows
    * [q_index_base, q_index_base + Lq) of a longer query; score_mod, mask_mod and the tile
-   * lists see the full-sequence row index.  Lets a caller run a query of more than 64 rows
-   * against a long KV cache as several decode calls.  A multiple of 64. */
+   * lists see the full-sequence row index.  Lets a caller run a query of more rows than one
+   * call takes against a long KV cache as several decode calls.  A multiple of 32. */
   int32_t q_index_base;
   int32_t pad_;
   /* flexattn_bwd only, optional (NULL = zero): cotangent of the lse2 output, [B,Hq,Lq] fp32.
@@ -226,8 +226,9 @@ int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* k, const vo
                  const void* o, const float* lse2, const void* d_o,
                  void* dq, void* dk, void* dv, void* workspace, flexattn_stream_t stream);
 
-/* Split-KV decode for short queries (Lq <= 64).  Replaces the same reference
- * functions as flexattn_fwd for the decode shapes of
+/* Split-KV decode for short queries: fp16 / bf16, D = Dv in {64, 128} with at most 64 query
+ * columns (query rows x query heads per KV head) or D = Dv = 256 with at most 32.  Replaces the
+ * same reference functions as flexattn_fwd for the decode shapes of
  * examples/benchmark_decoding.py:29-33.  num_splits <= 0 picks a default.  */
 size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32_t num_splits);
 int flexattn_decode(const FlexAttnParams* p, const void* q, const void* k, const void* v,

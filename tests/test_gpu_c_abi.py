@@ -72,7 +72,7 @@ def test_errors_launch_nothing(dev):
     p = _params(q, k, v, o)   # decode takes at most 64 query columns
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
     assert L.flexattn_decode(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, 2, ws.data_ptr(), _stream()) != 0
-    assert b"Lq <= 64" in L.flexattn_last_error()
+    assert b"at most 64 query columns" in L.flexattn_last_error()
     p.mask.kind = 1   # a bitmap mask without a bitmap
     assert L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), None, None, _stream()) != 0
     torch.cuda.synchronize()
