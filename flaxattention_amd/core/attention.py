@@ -275,7 +275,14 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
                 if lc is not lse2:
                     lse2[:, :, s0:s1] = lc
         else:
-            rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), None, _stream(q))
+            # few query tiles against many keys: with a workspace the library may split the call over the keys
+            ws = None
+            if plan.B * plan.Hq * ((plan.Lq + 127) // 128) < 128 and plan.Lkv >= 1024:
+                nbytes = L.flexattn_fwd_workspace_bytes(p)
+                if nbytes:
+                    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(),
+                                ws.data_ptr() if ws is not None else None, _stream(q))
             _lib.check(rc, "flexattn_fwd")
     return o, lse2
 

@@ -31,7 +31,10 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
 void* flex_decode_static_scratch(size_t* bytes);
 void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb);
 bool flex_simple_supported(const FlexAttnParams& p, int which);
-int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+int flex_simple_fwd_splits(const FlexAttnParams& p);
+size_t flex_simple_fwd_partial_bytes(const FlexAttnParams& p, int splits);
+int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
+                    void* partials, hipStream_t s);
 int flex_simple_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                     const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
 
@@ -109,9 +112,19 @@ extern "C" int flexattn_kernel_family(const FlexAttnParams* p, int32_t which) {
 
 static size_t lse_bytes(const FlexAttnParams* p) { return ((size_t)p->B * p->Hq * p->Lq * sizeof(float) + 255) / 256 * 256; }
 
+// the two passes of the parity numerics hand the log-sum-exp over in lse2, or in the workspace when the caller wants
+// no lse2; the space is reserved whenever the flag is set
+static size_t fwd_lse_bytes(const FlexAttnParams* p) {
+  return ((p->flags & FLEX_PARITY) && !(p->flags & FLEX_UNROUNDED)) ? lse_bytes(p) : 0;
+}
+
 extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
-  // the two passes of the parity numerics hand the log-sum-exp over in lse2, or here when the caller wants no lse2
-  return (p && (p->flags & FLEX_PARITY) && !(p->flags & FLEX_UNROUNDED)) ? lse_bytes(p) : 0;
+  if (!p) return 0;
+  size_t n = fwd_lse_bytes(p);
+  // the simple matrix-core kernels split the keys of a call with few query tiles over several workgroups, whose
+  // partial results live here
+  if (wants_fused(p) && flex_simple_supported(*p, 0)) n += flex_simple_fwd_partial_bytes(*p, flex_simple_fwd_splits(*p));
+  return n;
 }
 
 extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
@@ -129,7 +142,10 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
       if (!workspace) { flex_set_error("flexattn_fwd: FLEX_PARITY needs lse2 or a workspace of flexattn_fwd_workspace_bytes()"); return 1; }
       lse2 = (float*)workspace;
     }
-    if (int rcs = flex_simple_fwd(ps, q, k, v, o, lse2, s)) return rcs;
+    // with a workspace, a call with few query tiles is split over the keys (the partials follow the log-sum-exp space)
+    const int splits = workspace ? flex_simple_fwd_splits(ps) : 1;
+    void* partials = splits > 1 ? (char*)workspace + fwd_lse_bytes(p) : nullptr;
+    if (int rcs = flex_simple_fwd(ps, q, k, v, o, lse2, splits, partials, s)) return rcs;
     return check_launch("flexattn_fwd");
   }
   const bool fused = wants_fused(p) && flex_mfma_fwd_supported(*p);

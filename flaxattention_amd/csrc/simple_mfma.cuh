@@ -13,6 +13,7 @@
 // per SIMD (the widest instantiations hold more than 400 registers, accumulators in AGPRs).
 #pragma once
 #include "mfma_common.cuh"
+#include "decode.cuh"  // decode_combine_kernel merges the partials of a forward over split key ranges
 
 namespace flex {
 
@@ -210,10 +211,15 @@ struct SimpleSteps {
 //   kSimpleLse      first pass of the parity numerics: only lse2 (unrounded exponentials summed in fp32), V is not read
 //   kSimpleNorm     second pass: P = 2^(x - lse2) is the normalised probability, rounded to T for the product with V
 enum { kSimpleOnePass = 0, kSimpleLse = 1, kSimpleNorm = 2 };
+// Split-KV: with gridDim.y > 1 workgroup (x, y) takes share y of its query tile's key steps and leaves an unnormalised
+// partial (O, m, l) per row in o_part / ml_part, in the layout decode_combine_kernel merges (kSimpleLse: only (m, l);
+// kSimpleNorm: the partial outputs add up, written with m = 0 and l = 1 for share 0, l = 0 for the others).  For calls
+// whose query tiles alone would leave most compute units without a workgroup.
 template <typename T, int D, int KIND, int PASS>
 __global__ __launch_bounds__(256) void simple_fwd_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                          const T* __restrict__ k, const T* __restrict__ v,
-                                                         T* __restrict__ o, float* __restrict__ lse2) {
+                                                         T* __restrict__ o, float* __restrict__ lse2,
+                                                         float* __restrict__ o_part, float* __restrict__ ml_part) {
   typedef SimpleOps<T, D> Ops;
   constexpr int DB = D / 32, ROWE = Ops::ROWE;
   __shared__ __align__(16) T Ks[kSimpleStep * ROWE];
@@ -227,6 +233,7 @@ __global__ __launch_bounds__(256) void simple_fwd_kernel(FlexAttnParams p, const
   const int qt = nqt - 1 - rank;  // late query tiles see the most keys under causal masks
   const int h = bh % p.Hq, b = bh / p.Hq, hk = h / (p.Hq / p.Hkv);
   const int q_row = qt * kSimpleQTile + w * 32 + i32;
+  const bool wave_has_rows = __builtin_amdgcn_readfirstlane(q_row - i32) < p.Lq;  // short queries: decode shapes
   const int64_t row_id = ((int64_t)b * p.Hq + h) * p.Lq + min(q_row, p.Lq - 1);
   const bool round_s = Ops::kRounds && (p.flags & FLEX_ROUND_S);
 
@@ -238,6 +245,9 @@ __global__ __launch_bounds__(256) void simple_fwd_kernel(FlexAttnParams p, const
   st.init(tl.kv_num, tl.kv_idx, tl.full_kv_num, tl.full_kv_idx,
           (b * tl.stride_b + h * tl.stride_h) * tl.n_q_blocks + qt, tl.n_kv_blocks, tl.kv_block, p.Lkv, p.mask);
   const int nt = st.count(), n_full_t = st.full_steps();
+  const int nsplit = gridDim.y, split = blockIdx.y;
+  const int per = (nt + nsplit - 1) / nsplit;
+  const int it0 = split * per, it1 = min(it0 + per, nt);  // this workgroup's steps
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
@@ -257,22 +267,23 @@ __global__ __launch_bounds__(256) void simple_fwd_kernel(FlexAttnParams p, const
   }
 
   RowTile<T, D> kt, vt;
-  int s_cur = nt > 0 ? st.at(0) : 0;
-  if (nt > 0) {
+  int s_cur = it0 < it1 ? st.at(it0) : 0;
+  if (it0 < it1) {
     kt.load(kbase, p.k_stride[2], s_cur * kSimpleStep, p.Lkv - 1, tid);
     if constexpr (PASS != kSimpleLse) vt.load(vbase, p.v_stride[2], s_cur * kSimpleStep, p.Lkv - 1, tid);
   }
-  for (int it = 0; it < nt; it++) {
+  for (int it = it0; it < it1; it++) {
     const int kv0 = s_cur * kSimpleStep;
     __syncthreads();  // the previous step's reads are done
     kt.store(Ks, tid);
     if constexpr (PASS != kSimpleLse) vt.store(Vs, tid);
     __syncthreads();
-    if (it + 1 < nt) {
+    if (it + 1 < it1) {
       s_cur = st.at(it + 1);
       kt.load(kbase, p.k_stride[2], s_cur * kSimpleStep, p.Lkv - 1, tid);
       if constexpr (PASS != kSimpleLse) vt.load(vbase, p.v_stride[2], s_cur * kSimpleStep, p.Lkv - 1, tid);
     }
+    if (!wave_has_rows) continue;  // a wave past the last query row only helps to stage the tiles
     const bool masked = (it >= n_full_t) || (kv0 + kSimpleStep > p.Lkv);
     int cls = kBlockAll;
     if (masked) {
@@ -314,6 +325,28 @@ __global__ __launch_bounds__(256) void simple_fwd_kernel(FlexAttnParams p, const
   }
 
   const float l_tot = PASS == kSimpleNorm ? 1.f : xhalf_sum(l_run);
+  if (nsplit > 1) {
+    if (q_row < p.Lq) {
+      const int64_t at = (int64_t)split * p.B * p.Hq * p.Lq + row_id;
+      if (g == 0) {
+        ml_part[at * 2] = PASS == kSimpleNorm ? 0.f : m_run;
+        ml_part[at * 2 + 1] = PASS == kSimpleNorm ? (split == 0 ? 1.f : 0.f) : l_tot;
+      }
+      if constexpr (PASS != kSimpleLse) {
+        float* op = o_part + at * D + 4 * g;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+          for (int rr = 0; rr < 4; rr++) {
+            float4_t acc4;
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc4[e] = oacc[db][4 * rr + e];
+            *reinterpret_cast<float4_t*>(op + 32 * db + 8 * rr) = acc4;
+          }
+      }
+    }
+    return;
+  }
   const float inv = PASS == kSimpleNorm ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);
   if (q_row < p.Lq) {
     if constexpr (PASS != kSimpleLse) {
@@ -614,19 +647,36 @@ struct SimpleArgs {
   float *lse2_out, *delta;
   hipStream_t s;
   bool bwd;
+  // forward over split key ranges: shares per query tile (1 = none) and where their partial (O, m, l) go
+  int splits;
+  float *o_part, *ml_part;
 };
 
 template <typename T, int D, int KIND> void simple_launch_fwd(const FlexAttnParams& p, const SimpleArgs& a) {
-  const dim3 grid((p.Lq + kSimpleQTile - 1) / kSimpleQTile * p.Hq * p.B), block(256);
+  const int splits = a.splits > 1 ? a.splits : 1;
+  const dim3 grid((p.Lq + kSimpleQTile - 1) / kSimpleQTile * p.Hq * p.B, splits), block(256);
   const T *q = (const T*)a.q, *k = (const T*)a.k, *v = (const T*)a.v;
+  // split key ranges: every pass is followed by the merge of its partials (one wave per row)
+  auto merge = [&](T* o, float* lse2) {
+    if (splits == 1) return;
+    const int64_t rows = (int64_t)p.B * p.Hq * p.Lq;
+    hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, a.s, p, a.o_part, a.ml_part,
+                       splits, o, lse2);
+  };
   if constexpr (SimpleOps<T, D>::kRounds) {  // the parity numerics exist where something is rounded
     if (p.flags & FLEX_PARITY) {
-      hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleLse>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out);
-      hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleNorm>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out);
+      hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleLse>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out,
+                         a.o_part, a.ml_part);
+      merge(nullptr, a.lse2_out);
+      hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleNorm>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out,
+                         a.o_part, a.ml_part);
+      merge((T*)a.out, nullptr);
       return;
     }
   }
-  hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleOnePass>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out);
+  hipLaunchKernelGGL((simple_fwd_kernel<T, D, KIND, kSimpleOnePass>), grid, block, 0, a.s, p, q, k, v, (T*)a.out, a.lse2_out,
+                     a.o_part, a.ml_part);
+  merge((T*)a.out, a.lse2_out);
 }
 template <typename T, int D, int KIND> void simple_launch_bwd(const FlexAttnParams& p, const SimpleArgs& a) {
   const dim3 qgrid((p.Lq + kSimpleQTile - 1) / kSimpleQTile * p.Hq * p.B);

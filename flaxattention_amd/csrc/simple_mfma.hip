@@ -47,7 +47,27 @@ static int dispatch(const FlexAttnParams& p, const SimpleArgs& a) {
   return rc;
 }
 
-int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
+// Shares of the key steps a forward call is split into (1 = none): calls whose query tiles alone would leave most
+// compute units without a workgroup -- few rows against a long key sequence -- are split until there is about one
+// workgroup per compute unit, with at least 16 steps of 32 keys each.
+int flex_simple_fwd_splits(const FlexAttnParams& p) {
+  const int64_t wgs = (int64_t)((p.Lq + kSimpleQTile - 1) / kSimpleQTile) * p.Hq * p.B;
+  if (wgs >= 128) return 1;
+  const int steps = (p.Lkv + kSimpleStep - 1) / kSimpleStep;
+  int s = (int)(256 / wgs);
+  if (s > steps / 16) s = steps / 16;
+  if (s > 64) s = 64;  // the merge kernel takes one split per lane
+  return s < 2 ? 1 : s;
+}
+// bytes of the partial (O, m, l) of a split forward
+size_t flex_simple_fwd_partial_bytes(const FlexAttnParams& p, int splits) {
+  if (splits <= 1) return 0;
+  return ((size_t)p.B * p.Hq * p.Lq * splits * (p.D + 2) * sizeof(float) + 255) / 256 * 256;
+}
+
+// partials: nullptr for one pass over all keys, else flex_simple_fwd_partial_bytes(p, splits) bytes
+int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
+                    void* partials, hipStream_t s) {
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) {
     flex_set_error("matrix-core forward needs 16-byte aligned tensors");
     return 1;
@@ -58,6 +78,16 @@ int flex_simple_fwd(const FlexAttnParams& p, const void* q, const void* k, const
   }
   SimpleArgs a = {};
   a.q = q; a.k = k; a.v = v; a.out = o; a.lse2_out = lse2; a.s = s; a.bwd = false;
+  a.splits = 1;
+  if (splits > 1 && partials) {
+    if ((uintptr_t)partials & 15) {
+      flex_set_error("matrix-core forward needs a 16-byte aligned workspace");
+      return 1;
+    }
+    a.splits = splits;
+    a.o_part = (float*)partials;
+    a.ml_part = a.o_part + (size_t)p.B * p.Hq * p.Lq * splits * p.D;
+  }
   return dispatch(p, a);
 }
 

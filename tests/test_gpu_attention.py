@@ -255,6 +255,40 @@ def test_wide_heads_gqa_ragged_padded_bitmap(dev):
     run(dev, torch.float16, 2, 3, 3, 100, 150, 224, Dv=200, mask=weird, omask=weird, strict=False)
 
 
+SPLIT_CASES = [
+    # name, dtype, D, B, Hq, Hkv, Lq, kernel_options
+    ("f32-64", torch.float32, 64, 1, 2, 2, 5, None),
+    ("f32-128-gqa-two-tiles", torch.float32, 128, 1, 4, 2, 130, None),
+    ("bf16-192-parity", torch.bfloat16, 192, 2, 2, 2, 3, None),
+    ("f16-192-fast", torch.float16, 192, 1, 3, 3, 33, None),
+    ("f16-256-forward-kernel", torch.float16, 256, 1, 2, 2, 40, {"decode": False}),
+    ("bf16-256-fast-no-lists", torch.bfloat16, 256, 1, 2, 1, 17, {"numerics": "fast", "tile_lists": False, "decode": False}),
+]
+
+
+@pytest.mark.parametrize("name,dtype,D,B,Hq,Hkv,Lq,opts", SPLIT_CASES, ids=[c[0] for c in SPLIT_CASES])
+def test_forward_split_over_keys(dev, name, dtype, D, B, Hq, Hkv, Lq, opts):
+    """Few query rows against many keys on the simple matrix-core kernels: the forward is split over the keys and
+    merged (one-pass and both passes of the parity numerics), ALiBi + offset-causal with a ragged key length; the
+    first rows see no key at all (lse -inf, O = 0)."""
+    from flaxattention_amd import _lib
+    from flaxattention_amd.core.attention import _make_plan
+    print(f"case split forward {name}", flush=True)
+    Lkv, off = 2100, 2100 - Lq - 2   # row i sees keys <= i + off: the window ends two keys before the end
+    mask, omask = offset_causal_mask(off), o_offset_causal(off)
+    run(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, score=generate_alibi_bias(Hq, -1.0), oscore=o_alibi_config(Hq),
+        mask=mask, omask=omask, strict=False, opts=opts)
+    dead_off = -2                     # rows 0 and 1 see nothing
+    run(dev, dtype, B, Hq, Hkv, Lq, Lkv, D, mask=offset_causal_mask(dead_off), omask=o_offset_causal(dead_off),
+        strict=False, opts=opts, grad=False)
+    # the library does ask for room for the partial results of such a call
+    q, k, v = (t.to(dev) for t in seeded_qkv(B, Hq, Hkv, Lq, Lkv, D, dtype))
+    plan = _make_plan(q, k, v, None, None, None, 1.0, opts)
+    o = torch.empty_like(q)
+    nbytes = _lib.lib().flexattn_fwd_workspace_bytes(plan.params(q, k, v, o))
+    assert nbytes >= 2 * B * Hq * Lq * (D + 2) * 4
+
+
 # ---- faithful kernels, 16-bit, every functor ----
 SCORES = [
     ("identity", None, None),
