@@ -36,9 +36,16 @@ selects numerics here:
                         in the input dtype)
     {"backend": "generic" | "auto"}
     {"decode": bool}      split-KV decode kernel on / off; by default it is used
-                          whenever it applies (fp16/bf16, D = Dv in {64, 128},
-                          at most 64 query rows per KV head, at least 512 keys)
+                          whenever it applies (fp16/bf16, D = Dv in {64, 128} with
+                          at most 64 query rows per KV head or D = Dv = 256 with at
+                          most 32, at least 512 keys); True also runs longer queries
+                          through it, in chunks of that many rows
     {"decode_splits": n}  force the split-KV decode kernel with n splits
+    {"split_kv": bool}    False: the forward kernel never splits a call over the keys
+                          (by default it does when the query tiles alone are fewer
+                          workgroups than the GPU has compute units); the result of a
+                          (batch, head) pair then does not depend on how many pairs
+                          the call has, bit for bit
     {"pad_head_dim": bool}  inputs whose head sizes are not among those of the matrix-core kernels
                           (D = Dv in {64, 128}, 16-bit inputs also {192, 256}) but no larger are
                           zero-padded to the next of those (default True)
@@ -115,6 +122,7 @@ class _Plan:
         # decode_splits: > 0 = decode kernel with that many splits, < 0 = decode kernel with the
         # library's default split count, 0 = forward kernel
         self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
+        self.split_kv = True    # the forward kernel may split a call with few query tiles over the keys
         self.lists = None       # tile lists for the forward / decode kernels
         self.lists_bwd = None   # tile lists for the backward kernels
         self.keep = [mask.bits, score.mul, score.add]
@@ -175,6 +183,7 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
     if numerics == "unrounded":
         flags = (flags & ~(_lib.FLAG_ROUND_S | _lib.FLAG_STRICT)) | _lib.FLAG_UNROUNDED
     plan = _Plan(q, k, v, score, mask, block_mask, scale, flags, True, _decode_choice(q, k, v, score, flags, opts))
+    plan.split_kv = bool(opts.get("split_kv", True))
     # tile lists at the fused kernels' granularity (skipped for a mask that hides nothing)
     if not mask.is_noop() and opts.get("tile_lists", True) and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC)):
         holder = block_mask if block_mask is not None else _holder_for(mask)
@@ -208,13 +217,10 @@ def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
         return -1   # the library reports what does not fit
     if not ok:
         return 0
-    cols = _decode_columns(D)
-    if G * Lq <= cols:
-        return -1 if k.shape[2] >= 512 else 0
-    # up to four calls' worth of rows against a long KV cache: a few decode passes over the cache beat a forward
-    # grid that would leave most compute units without a workgroup (one per 128 query rows and head)
-    few_workgroups = B * Hq * ((Lq + 127) // 128) < 256
-    return -1 if (G == 1 and Lq <= 4 * cols and k.shape[2] >= 4096 and few_workgroups) else 0
+    # more rows than one decode call takes: the forward kernel, which splits a call with few query tiles over the keys
+    # (one pass over the KV cache; measured faster than several decode calls of 64 rows: 124 us against 212 us for 256
+    # rows x 16384 keys); {"decode": True} still runs such a query through the decode kernel in chunks
+    return -1 if (G * Lq <= _decode_columns(D) and k.shape[2] >= 512) else 0
 
 
 def _decode_columns(D: int) -> int:
@@ -277,7 +283,7 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
         else:
             # few query tiles against many keys: with a workspace the library may split the call over the keys
             ws = None
-            if plan.B * plan.Hq * ((plan.Lq + 127) // 128) < 128 and plan.Lkv >= 1024:
+            if plan.split_kv and plan.B * plan.Hq * ((plan.Lq + 127) // 128) < 256 and plan.Lkv >= 1024:
                 nbytes = L.flexattn_fwd_workspace_bytes(p)
                 if nbytes:
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)

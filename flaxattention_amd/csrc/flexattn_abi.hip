@@ -18,7 +18,10 @@ int flex_generic_fwd(const FlexAttnParams& p, const void* q, const void* k, cons
 int flex_generic_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const float* lse2, const void* d_o,
                      void* dq, void* dk, void* dv, float* delta, hipStream_t s);
 bool flex_mfma_fwd_supported(const FlexAttnParams& p);
-int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s);
+int flex_mfma_fwd_splits(const FlexAttnParams& p);
+size_t flex_mfma_fwd_partial_bytes(const FlexAttnParams& p, int splits);
+int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
+                  void* partials, hipStream_t s);
 bool flex_mfma_bwd_supported(const FlexAttnParams& p);
 size_t flex_mfma_bwd_workspace(const FlexAttnParams& p);
 int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
@@ -121,9 +124,10 @@ static size_t fwd_lse_bytes(const FlexAttnParams* p) {
 extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
   if (!p) return 0;
   size_t n = fwd_lse_bytes(p);
-  // the simple matrix-core kernels split the keys of a call with few query tiles over several workgroups, whose
+  // the matrix-core forward kernels split the keys of a call with few query tiles over several workgroups, whose
   // partial results live here
   if (wants_fused(p) && flex_simple_supported(*p, 0)) n += flex_simple_fwd_partial_bytes(*p, flex_simple_fwd_splits(*p));
+  else if (wants_fused(p) && flex_mfma_fwd_supported(*p)) n += flex_mfma_fwd_partial_bytes(*p, flex_mfma_fwd_splits(*p));
   return n;
 }
 
@@ -155,7 +159,10 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
       if (!workspace) { flex_set_error("flexattn_fwd: FLEX_PARITY needs lse2 or a workspace of flexattn_fwd_workspace_bytes()"); return 1; }
       lse2 = (float*)workspace;
     }
-    rc = flex_mfma_fwd(pr, q, k, v, o, lse2, s);
+    // with a workspace, a call with few query tiles is split over the keys (the partials follow the log-sum-exp space)
+    const int splits = workspace ? flex_mfma_fwd_splits(pr) : 1;
+    void* partials = splits > 1 ? (char*)workspace + fwd_lse_bytes(p) : nullptr;
+    rc = flex_mfma_fwd(pr, q, k, v, o, lse2, splits, partials, s);
   } else {
     rc = flex_generic_fwd(pr, q, k, v, o, lse2, s);
   }

@@ -21,6 +21,7 @@
 //   layout; V^T fragments come from transposing LDS reads)
 #pragma once
 #include "mfma_common.cuh"
+#include "decode.cuh"  // decode_combine_kernel merges the partials of a forward over split key ranges
 
 namespace flex {
 
@@ -44,7 +45,12 @@ enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2, kFwdHiLo = 3 };
 template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
 __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
-                                                           T* __restrict__ o, float* __restrict__ lse2) {
+                                                           T* __restrict__ o, float* __restrict__ lse2,
+                                                           float* __restrict__ o_part, float* __restrict__ ml_part) {
+  // Split-KV: with gridDim.y > 1 workgroup (x, y) visits share y of its query tile's key tiles and leaves an
+  // unnormalised partial (O, m, l) per row in o_part / ml_part, in the layout decode_combine_kernel merges (kFwdLse:
+  // only (m, l); kFwdNorm: the partial outputs add up, written with m = 0 and l = 1 for share 0, l = 0 for the
+  // others).  For calls whose query tiles alone would leave most compute units without a workgroup.
   typedef typename Frag<T>::vec8 vec8;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   constexpr int RQ = 1, BM = kFwdBM, BN = kFwdBN;
@@ -103,6 +109,10 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
     if (!full_idx) return nt - 1 - it;
     return uniform_ld(it < n_part ? part_idx + (n_part - 1 - it) : full_idx + (n_full - 1 - (it - n_part)));
   };
+  // this workgroup's share of the visits: [it0, it1)
+  const int nsplit = gridDim.y, split = blockIdx.y;
+  const int per = (nt + nsplit - 1) / nsplit;
+  const int it0 = split * per, it1 = min(it0 + per, nt);
 
   const T* kbase = k + b * p.k_stride[0] + hk * p.k_stride[1];
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
@@ -172,25 +182,29 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   // (fp16 tops out at 65504; sums are kept in fp32) or when a row that has accumulated nothing sees a block whose
   // exponentials are all below kPTiny
   constexpr float kPGuard = 32768.f, kPTiny = 1.f / 64.f;
-  int t_cur = nt > 0 ? tile_at(0) : 0;
-  int t_nxt = nt > 1 ? tile_at(1) : 0;
-  // prologue: tile 0 into stage 0, tile 1 into registers
-  if (nt > 0) load_tile(t_cur * BN);
+  int t_cur = it0 < it1 ? tile_at(it0) : 0;
+  int t_nxt = it0 + 1 < it1 ? tile_at(it0 + 1) : 0;
+  // prologue: the first tile into its stage, the second into registers
+  int any_tile = it0 < it1;
+  if (any_tile) load_tile(t_cur * BN);
   // Unconditional, and as an instruction the compiler's wait-count pass sees: the Q fragments (and tile 0) have
-  // arrived.  With the wait only inside the nt > 0 branch the pass carries "Q fragments may still be in flight" into
+  // arrived.  With the wait only inside the branch the pass carries "Q fragments may still be in flight" into
   // the loop and makes the first products of every tile wait for all outstanding loads, i.e. for the prefetch of the
-  // tile after next that was issued half a tile earlier.
+  // tile after next that was issued half a tile earlier.  The condition is made opaque in between so that the two
+  // branches around the wait are not merged into one (which moves a copy of the wait into each arm).
+  asm volatile("" : "+v"(any_tile));
+  any_tile = __builtin_amdgcn_readfirstlane(any_tile);
   __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  if (nt > 0) store_tile(0);
-  if (nt > 1) load_tile(t_nxt * BN);
+  if (any_tile) store_tile(it0 & 1);
+  if (it0 + 1 < it1) load_tile(t_nxt * BN);
   __syncthreads();
-  for (int it = 0; it < nt; it++) {
+  for (int it = it0; it < it1; it++) {
     const int kv0 = t_cur * BN;
     const bool masked = (it < n_part) || (kv0 + BN > p.Lkv);
     const T* Ks = Ksm[it & 1];
     const T* Vs = Vsm[PASS == kFwdLse ? 0 : (it & 1)];
     t_cur = t_nxt;
-    if (it + 2 < nt) t_nxt = tile_at(it + 2);
+    if (it + 2 < it1) t_nxt = tile_at(it + 2);
 
     // Each 32-row half of the tile is one online-softmax step.
 #pragma unroll
@@ -337,11 +351,11 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
         }
       }
       }  // block not entirely hidden
-      if (nb == 0 && it + 1 < nt) {
+      if (nb == 0 && it + 1 < it1) {
         // the other stage was last read before the previous barrier: refill it with the
         // tile prefetched into registers, then start fetching the one after
         store_tile((it + 1) & 1);
-        if (it + 2 < nt) load_tile(t_nxt * BN);
+        if (it + 2 < it1) load_tile(t_nxt * BN);
       }
     }
     __syncthreads();
@@ -352,6 +366,29 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   for (int a = 0; a < RQ; a++) {
     const int q_row = q_row0 + 32 * a;
     const float l_tot = PASS == kFwdNorm ? 1.f : xhalf_sum(l_run[a]);
+    if (nsplit > 1) {
+      // partial result of this share; a row that saw nothing here must not hold the merge's reference up: m = -inf
+      if (q_row < p.Lq) {
+        const int64_t at = ((int64_t)split * p.B * p.Hq + (int64_t)b * p.Hq + h) * p.Lq + q_row;
+        if (g == 0) {
+          ml_part[at * 2] = PASS == kFwdNorm ? 0.f : (l_tot > 0.f ? m_run[a] : -INFINITY);
+          ml_part[at * 2 + 1] = PASS == kFwdNorm ? (split == 0 ? 1.f : 0.f) : l_tot;
+        }
+        if constexpr (PASS != kFwdLse) {
+          float* op = o_part + at * D + 4 * g;
+#pragma unroll
+          for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int rr = 0; rr < 4; rr++) {
+              float4_t acc4;
+#pragma unroll
+              for (int e = 0; e < 4; e++) acc4[e] = oacc[a][db][4 * rr + e];
+              *reinterpret_cast<float4_t*>(op + 32 * db + 8 * rr) = acc4;
+            }
+        }
+      }
+      continue;
+    }
     const float inv = PASS == kFwdNorm ? 1.f : (l_tot > 0.f ? 1.f / l_tot : 0.f);  // kFwdNorm: P came normalised
     if (q_row < p.Lq) {
       if constexpr (PASS != kFwdLse) {
@@ -733,13 +770,24 @@ struct FwdArgs {
   void* o;
   float* lse2;
   hipStream_t s;
+  // forward over split key ranges: shares per query tile (1 = none) and where their partial (O, m, l) go
+  int splits;
+  float *o_part, *ml_part;
 };
 
+// one pass of the list-driven kernel; over split key ranges it is followed by the merge of the partials (one wave per
+// row), which writes `o` (unless null) and `lse2` (unless null)
 template <typename T, int D, int KIND, bool RS, bool BITS, int PASS>
 static void launch_list_kernel(const FlexAttnParams& p, const FwdArgs& a) {
-  dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B);
+  const int splits = a.splits > 1 ? a.splits : 1;
+  dim3 grid((p.Lq + kFwdBM - 1) / kFwdBM * p.Hq * p.B, splits);
   hipLaunchKernelGGL((fwd_mfma_kernel<T, D, KIND, RS, BITS, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
-                     (const T*)a.v, (T*)a.o, a.lse2);
+                     (const T*)a.v, (T*)a.o, a.lse2, a.o_part, a.ml_part);
+  if (splits > 1) {
+    const int64_t rows = (int64_t)p.B * p.Hq * p.Lq;
+    hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, a.s, p, a.o_part, a.ml_part,
+                       splits, PASS == kFwdLse ? (T*)nullptr : (T*)a.o, PASS == kFwdNorm ? (float*)nullptr : a.lse2);
+  }
 }
 
 template <typename T, int KIND, bool RS, bool TAIL>
@@ -775,7 +823,7 @@ static void launch_rs(const FlexAttnParams& p, const FwdArgs& a) {
   // longest one, which is what bounds a causal-like schedule.
   // (a table-reading score_mod stalls on its loads where the pipelined kernel has no slack: 128-row kernel)
   if constexpr (KIND != FLEX_SCORE_AFFINE && KIND != kScoreAffineMul && D == 64) {
-    if (!p.tiles.kv_num && mask_hides_nothing(p.mask)) {
+    if (!p.tiles.kv_num && mask_hides_nothing(p.mask) && a.splits <= 1) {
       const bool tail = p.Lkv % kFwdBN != 0, rs = (p.flags & FLEX_ROUND_S) != 0;
       if (rs && !tail) launch_pipe_kernel<T, KIND, true, false>(p, a);
       else if (rs) launch_pipe_kernel<T, KIND, true, true>(p, a);

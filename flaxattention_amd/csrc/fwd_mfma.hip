@@ -38,7 +38,27 @@ bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
   return !t.kv_num || (t.q_block == kFwdBM && t.kv_block == kFwdBN);
 }
 
-int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, hipStream_t s) {
+// Shares of the key tiles a forward call is split into (1 = none): calls whose query tiles alone would leave most
+// compute units without a workgroup (fewer than one per compute unit) -- few rows against a long key sequence -- are
+// split until there are about two workgroups per compute unit, with at least 8 tiles of 64 keys each.
+int flex_mfma_fwd_splits(const FlexAttnParams& p) {
+  const int64_t wgs = (int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B;
+  if (wgs >= 256) return 1;
+  const int tiles = (p.Lkv + kFwdBN - 1) / kFwdBN;
+  int s = (int)(512 / wgs);
+  if (s > tiles / 8) s = tiles / 8;
+  if (s > 64) s = 64;  // the merge kernel takes one split per lane
+  return s < 2 ? 1 : s;
+}
+// bytes of the partial (O, m, l) of a split forward
+size_t flex_mfma_fwd_partial_bytes(const FlexAttnParams& p, int splits) {
+  if (splits <= 1) return 0;
+  return ((size_t)p.B * p.Hq * p.Lq * splits * (p.D + 2) * sizeof(float) + 255) / 256 * 256;
+}
+
+// partials: nullptr for one pass over all keys, else flex_mfma_fwd_partial_bytes(p, splits) bytes
+int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
+                  void* partials, hipStream_t s) {
   if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)o) & 15) {
     flex_set_error("fused forward needs 16-byte aligned tensors");
     return 1;
@@ -47,7 +67,16 @@ int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const v
     flex_set_error("fused forward: the parity numerics need a log-sum-exp buffer (lse2 or workspace)");
     return 1;
   }
-  const FwdArgs a = {q, k, v, o, lse2, s};
+  FwdArgs a = {q, k, v, o, lse2, s, 1, nullptr, nullptr};
+  if (splits > 1 && partials) {
+    if ((uintptr_t)partials & 15) {
+      flex_set_error("fused forward needs a 16-byte aligned workspace");
+      return 1;
+    }
+    a.splits = splits;
+    a.o_part = (float*)partials;
+    a.ml_part = a.o_part + (size_t)p.B * p.Hq * p.Lq * splits * p.D;
+  }
   int rc = 1;
   if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_mfma_fwd_f16_64(p, a) : flex_mfma_fwd_f16_128(p, a);
   else rc = p.D == 64 ? flex_mfma_fwd_bf16_64(p, a) : flex_mfma_fwd_bf16_128(p, a);

@@ -206,8 +206,8 @@ int flexattn_block_mask_build(const FlexMask* mask, int32_t B, int32_t H,
 
 /* Forward.  With FLEX_PARITY and lse2 == NULL the log-sum-exp that the second pass reads is kept
  * in `workspace` (flexattn_fwd_workspace_bytes); otherwise workspace may be NULL.  A workspace
- * of that size also lets calls with few query rows against many keys (float32, or 16-bit head
- * sizes 192 / 256) be split over the keys, so that they fill the GPU; without one they run unsplit.
+ * of that size also lets the matrix-core kernels split calls with few query rows against many
+ * keys over the keys, so that they fill the GPU; without one such calls run unsplit.
  * Replaces math_attention (flaxattention/core/attention.py:67-106)
  * behind flax_attention (169-218) and mha_forward_kernel / _mha_forward
  * (flaxattention/kernel/attention.py:34-149, 260-335) behind

@@ -263,14 +263,20 @@ SPLIT_CASES = [
     ("f16-192-fast", torch.float16, 192, 1, 3, 3, 33, None),
     ("f16-256-forward-kernel", torch.float16, 256, 1, 2, 2, 40, {"decode": False}),
     ("bf16-256-fast-no-lists", torch.bfloat16, 256, 1, 2, 1, 17, {"numerics": "fast", "tile_lists": False, "decode": False}),
+    # the tuned 16-bit kernels (D 64 / 128)
+    ("f16-64", torch.float16, 64, 1, 2, 2, 100, None),
+    ("f16-64-short-no-lists", torch.float16, 64, 2, 2, 2, 7, {"decode": False, "tile_lists": False}),
+    ("bf16-128-parity-gqa", torch.bfloat16, 128, 1, 4, 2, 150, None),
+    ("bf16-64-fast", torch.bfloat16, 64, 1, 3, 3, 129, {"numerics": "fast"}),
+    ("f16-128-parity", torch.float16, 128, 1, 2, 2, 33, {"numerics": "parity", "decode": False}),
 ]
 
 
 @pytest.mark.parametrize("name,dtype,D,B,Hq,Hkv,Lq,opts", SPLIT_CASES, ids=[c[0] for c in SPLIT_CASES])
 def test_forward_split_over_keys(dev, name, dtype, D, B, Hq, Hkv, Lq, opts):
-    """Few query rows against many keys on the simple matrix-core kernels: the forward is split over the keys and
-    merged (one-pass and both passes of the parity numerics), ALiBi + offset-causal with a ragged key length; the
-    first rows see no key at all (lse -inf, O = 0)."""
+    """Few query rows against many keys: the matrix-core forward is split over the keys and merged (one-pass and both
+    passes of the parity numerics), ALiBi + offset-causal with a ragged key length; in a second call the first rows
+    see no key at all (lse -inf, O = 0)."""
     from flaxattention_amd import _lib
     from flaxattention_amd.core.attention import _make_plan
     print(f"case split forward {name}", flush=True)
@@ -287,6 +293,34 @@ def test_forward_split_over_keys(dev, name, dtype, D, B, Hq, Hkv, Lq, opts):
     o = torch.empty_like(q)
     nbytes = _lib.lib().flexattn_fwd_workspace_bytes(plan.params(q, k, v, o))
     assert nbytes >= 2 * B * Hq * Lq * (D + 2) * 4
+
+
+def test_forward_split_unrounded_equals_unsplit(dev):
+    """The "unrounded" numerics over split key ranges against the same call without a workspace (one pass over all
+    keys), through the C ABI; a causal bitmap-free band mask with tile lists."""
+    from flaxattention_amd import _lib
+    from flaxattention_amd.core.attention import _make_plan
+    L = _lib.lib()
+    B, H, Lq, Lkv, D = 1, 2, 90, 3000, 128
+    q, k, v = (t.to(dev) for t in seeded_qkv(B, H, H, Lq, Lkv, D, torch.bfloat16))
+    bm = fa.create_block_mask(offset_causal_mask(Lkv - Lq), B, H, Lq, Lkv, device=dev)
+    plan = _make_plan(q, k, v, generate_alibi_bias(H, -1.0), bm, None, D ** -0.5, {"numerics": "unrounded", "decode": False})
+    outs = []
+    stream = torch.cuda.current_stream().cuda_stream
+    for with_ws in (False, True):
+        o = torch.empty_like(q)
+        lse = torch.empty((B, H, Lq), dtype=torch.float32, device=dev)
+        p = plan.params(q, k, v, o)
+        n = L.flexattn_fwd_workspace_bytes(p)
+        assert n > 0
+        ws = torch.empty(n, dtype=torch.uint8, device=dev) if with_ws else None
+        rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse.data_ptr(),
+                            ws.data_ptr() if with_ws else None, stream)
+        assert rc == 0, L.flexattn_last_error()
+        torch.cuda.synchronize()
+        outs.append((o.float().cpu(), lse.cpu()))
+    assert max_abs(outs[0][0], outs[1][0]) <= 4e-3 and rel_l2(outs[1][0], outs[0][0]) <= 1e-3
+    assert max_abs(outs[0][1], outs[1][1]) <= 1e-4
 
 
 # ---- faithful kernels, 16-bit, every functor ----

@@ -67,8 +67,8 @@ def test_decode_256_wide_heads(dev, dtype, numerics, Lq, G, splits):
 
 
 def test_decode_256_wide_heads_choice_and_chunks(dev):
-    """D = 256 is routed to the decode kernel up to 32 columns per call; longer queries go in chunks of 32 rows; the
-    library refuses more than 32 columns in one call and the results agree with the forward kernel."""
+    """D = 256 is routed to the decode kernel up to 32 columns per call; longer queries go there in chunks of 32 rows
+    on request; the library refuses more than 32 columns in one call and the results agree with the forward kernel."""
     from flaxattention_amd.core.attention import _make_plan
     from flaxattention_amd import _lib
     B, H, Lq, Lkv, D = 1, 2, 80, 4096, 256
@@ -77,9 +77,10 @@ def test_decode_256_wide_heads_choice_and_chunks(dev):
     bm = fa.create_block_mask(mask, B, H, Lq, Lkv, device=dev)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     assert _make_plan(qd[:, :, :32], kd, vd, None, None, None, 0.0625, None).decode_splits < 0
-    assert _make_plan(qd, kd, vd, None, bm, None, 0.0625, None).decode_splits < 0          # 80 rows: three calls
-    assert _make_plan(qd, kd, vd, None, bm, None, 0.0625, {"decode": False}).decode_splits == 0
-    out, lse = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True)
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.0625, None).decode_splits == 0         # 80 rows: the forward kernel
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.0625, {"decode": True}).decode_splits < 0   # on request: three calls
+    out, lse = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True,
+                                 kernel_options={"decode": True})
     want, want_lse = ref_attention(q, k, v, o_alibi_config(H), omask, strict=True, return_lse=True)
     a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
     print(f"  chunked decode at D=256 O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
@@ -176,7 +177,7 @@ def test_decode_is_chosen_automatically(dev):
 
 
 def test_decode_in_chunks_of_64_rows(dev):
-    """Queries of 65..256 rows against a long KV cache run as several decode calls, each seeing its
+    """On request ({"decode": True}) queries of more than 64 rows run as several decode calls, each seeing its
     row offset in score_mod, mask_mod and the tile lists (ALiBi + offset-causal, ragged last chunk)."""
     from flaxattention_amd.core.attention import _make_plan
     B, H, Lq, Lkv, D = 1, 2, 160, 4096, 64
@@ -184,9 +185,10 @@ def test_decode_in_chunks_of_64_rows(dev):
     mask, omask = offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq)
     bm = fa.create_block_mask(mask, B, H, Lq, Lkv, device=dev)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
-    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, None).decode_splits < 0          # chosen automatically
-    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, {"decode": False}).decode_splits == 0
-    out, lse = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True)
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, None).decode_splits == 0         # by default: the forward kernel
+    assert _make_plan(qd, kd, vd, None, bm, None, 0.125, {"decode": True}).decode_splits < 0
+    out, lse = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True,
+                                 kernel_options={"decode": True})
     want, want_lse = ref_attention(q, k, v, o_alibi_config(H), omask, strict=True, return_lse=True)
     a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
     print(f"  chunked decode O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
