@@ -262,8 +262,8 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
             if plan.Lq <= rows:
                 chunks = [(0, plan.Lq, q, o, lse2, p)]
             else:
-                # a longer query goes through the decode kernel 64 (D = 256: 32) rows at a time (chunking is
-                # only chosen without GQA packing), each call seeing its row offset
+                # on request ({"decode": True}) a longer query goes through the decode kernel 64 (D = 256: 32)
+                # columns at a time, each call seeing its row offset
                 chunks = []
                 for s0 in range(0, plan.Lq, rows):
                     s1 = min(s0 + rows, plan.Lq)
