@@ -85,6 +85,9 @@ class Prepared:
         self.dq, self.dk, self.dv = torch.empty_like(self.q), torch.empty_like(self.k), torch.empty_like(self.v)
         self.p = self.plan.params(self.q, self.k, self.v, self.o)
         self.ws = torch.empty(max(self.L.flexattn_bwd_workspace_bytes(self.p), 256), dtype=torch.uint8, device=dev)
+        # forward workspace as the front-end passes it: lets the library split a call with few query tiles over the keys
+        n = self.L.flexattn_fwd_workspace_bytes(self.p)
+        self.fws = torch.empty(n, dtype=torch.uint8, device=dev) if n else None
         self.splits = decode_splits
         if decode_splits:
             n = self.L.flexattn_decode_workspace_bytes(self.p, decode_splits)
@@ -107,7 +110,8 @@ class Prepared:
 
     def fwd(self):
         t = self.ptr
-        rc = self.L.flexattn_fwd(self.p, t["q"], t["k"], t["v"], t["o"], t["lse"], None, self.stream)
+        rc = self.L.flexattn_fwd(self.p, t["q"], t["k"], t["v"], t["o"], t["lse"],
+                                 self.fws.data_ptr() if self.fws is not None else None, self.stream)
         if rc:
             self._lib.check(rc, "flexattn_fwd")
 
