@@ -239,7 +239,7 @@ extern "C" int flexattn_decode_static(const FlexAttnParams* p, const void* q, co
 static int decode_checked(const FlexAttnParams* p, const void* q, const void* k, const void* v, void* o, float* lse2,
                           int32_t num_splits, void* workspace, flexattn_stream_t stream) {
   if (p->flags & FLEX_UNROUNDED) { flex_set_error("flexattn_decode: FLEX_UNROUNDED is served by flexattn_fwd (the decode kernel carries P in one part)"); return 1; }
-  if (p->q_index_base < 0 || p->q_index_base % 32 != 0) { flex_set_error("flexattn_decode: q_index_base must be a non-negative multiple of 32 (got %d)", p->q_index_base); return 1; }
+  if (p->q_index_base < 0) { flex_set_error("flexattn_decode: q_index_base must not be negative (got %d)", p->q_index_base); return 1; }
   if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
   if (!flex_decode_supported(*p)) {
     flex_set_error("flexattn_decode: needs fp16/bf16 and D == Dv in {64,128} with at most 64 query columns or D == Dv == 256 with at most 32 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);

@@ -156,7 +156,7 @@ typedef struct FlexAttnParams {
   /* flexattn_decode only (0 elsewhere): the query tensor passed in is rows
    * [q_index_base, q_index_base + Lq) of a longer query; score_mod, mask_mod and the tile
    * lists see the full-sequence row index.  Lets a caller run a query of more rows than one
-   * call takes against a long KV cache as several decode calls.  A multiple of 32. */
+   * call takes against a long KV cache as several decode calls.  Not negative. */
   int32_t q_index_base;
   int32_t pad_;
   /* flexattn_bwd only, optional (NULL = zero): cotangent of the lse2 output, [B,Hq,Lq] fp32.

@@ -198,6 +198,27 @@ def test_decode_in_chunks_of_64_rows(dev):
     assert max_abs(out.cpu(), ref.cpu()) <= 2e-3
 
 
+def test_decode_in_chunks_with_gqa_packing(dev):
+    """{"decode": True} with several query heads per KV head: a call takes 64 / G rows, so the chunks start at row
+    offsets that are multiples of 16 here (sink + window band mask, ALiBi, bf16 in its default numerics)."""
+    from flaxattention_amd.core.common import MaskMod
+    B, Hq, Hkv, Lq, Lkv, D = 2, 8, 2, 82, 2047, 128
+    q, k, v = seeded_qkv(B, Hq, Hkv, Lq, Lkv, D, torch.bfloat16)
+    off = Lkv - Lq
+    mask = MaskMod(lo=0, hi=700, sink=4, q_offset=off, name="decode_sink_window")
+    def omask(b, h, q_idx, kv_idx):
+        d = q_idx + off - kv_idx
+        return ((d >= 0) & (d <= 700)) | ((kv_idx <= 4) & (d >= 0))   # MaskMod: keys 0 .. sink stay visible
+    bm = fa.create_block_mask(mask, B, Hq, Lq, Lkv, device=dev)
+    out, lse = fa.flax_attention(q.to(dev), k.to(dev), v.to(dev), score_mod=generate_alibi_bias(Hq, -1.0), block_mask=bm,
+                                 enable_gqa=True, return_lse=True, kernel_options={"decode": True})
+    want, want_lse = ref_attention(q, k, v, o_alibi_config(Hq), omask, strict=True, return_lse=True)
+    a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
+    print(f"  chunked decode with GQA O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
+    assert a <= 2e-2 and r <= 1e-3
+    assert max_abs(lse.cpu(), want_lse) <= 2e-2
+
+
 @pytest.mark.parametrize("Lq", [1, 200])
 def test_calls_replay_from_a_captured_graph(dev, Lq):
     """Nothing on the path synchronises, allocates outside the caller's allocator or records a memset, so a serving
