@@ -7,7 +7,7 @@
 //
 // Two kernels.  fwd_mfma_kernel (any supported D, tile lists or not): one workgroup
 // (4 waves) per 128 query rows of one (batch, head), one 32-row block per wave; KV tiles of
-// 64 rows go through two LDS stages (register-prefetched one tile ahead, one workgroup
+// 64 rows go through two LDS stages (fetched global -> LDS directly one tile ahead, one workgroup
 // barrier per tile).  fwd_pipe_kernel (D = 64, no tile lists, a mask that hides nothing): 256 query rows per
 // workgroup, two blocks per wave, software-pipelined (see there).
 // Per 32-key step and 32-row block:
@@ -56,13 +56,19 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   constexpr int RQ = 1, BM = kFwdBM, BN = kFwdBN;
   constexpr int DS = D / 16;     // k-steps of the Q.K^T product
   constexpr int DB = D / 32;     // 32-row blocks of O^T
-  constexpr int ROWE = D + 8;    // LDS row length in elements (16 B of padding)
   constexpr int CPR = D / 8;     // 16-byte chunks per row
-  constexpr int NLD = BN * CPR / 256;  // chunks per thread per tile
-  // two LDS stages: while one tile is consumed the next one is written, so a
-  // single workgroup barrier per tile suffices
-  __shared__ __align__(16) T Ksm[2][BN * ROWE];
-  __shared__ __align__(16) T Vsm[PASS == kFwdLse ? 1 : 2][PASS == kFwdLse ? 8 : BN * ROWE];
+  constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
+  constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor (a wave fills 16 rows = one swizzle period)
+  static_assert((BN / 4) == 16, "a wave's share of a tile is one swizzle period");
+  // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled rows): while one
+  // tile is consumed the next one lands, one workgroup barrier per tile.  Each stage is a variable of its own and
+  // every access names its stage at compile time (the tile loop is unrolled by two): only then can the compiler
+  // tell that a read of one stage need not wait for the fetch into the other.
+  constexpr int kVElems = PASS == kFwdLse ? 8 : BN * D;
+  __shared__ __align__(16) T Ksm0[BN * D];
+  __shared__ __align__(16) T Ksm1[BN * D];
+  __shared__ __align__(16) T Vsm0[kVElems];
+  __shared__ __align__(16) T Vsm1[kVElems];
 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int i32 = lane & 31, g = lane >> 5, i16 = lane & 15;
@@ -118,44 +124,67 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   const T* vbase = v + b * p.v_stride[0] + hk * p.v_stride[1];
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
 
-  u32x4 kreg[NLD], vreg[NLD];
-  // the per-lane part of a load address (row inside the tile, chunk) is the same for every tile: kept as byte
-  // offsets from the tile's first row, whose address is wave-uniform
-  uint32_t klo[NLD], vlo[NLD];
+  // tile fetch: wave w fills rows [16w, 16w + 16) of the K and the V tile, RPI rows per instruction; the lane that
+  // fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row.  The per-lane part of a fetch address (row
+  // inside the swizzle period, swizzled chunk) is the same for every tile: kept as byte offsets from a wave-uniform
+  // row address.
+  const int fill_row = lane / CPR, fill_pos = lane % CPR;
+  const int wu = __builtin_amdgcn_readfirstlane(w);
+  uint32_t koff[NI], voff[NI];
 #pragma unroll
-  for (int j = 0; j < NLD; j++) {
-    const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-    klo[j] = (uint32_t)((r * ks2 + cc * 8) * (int64_t)sizeof(T));
-    vlo[j] = (uint32_t)((r * vs2 + cc * 8) * (int64_t)sizeof(T));
+  for (int j = 0; j < NI; j++) {
+    const int row = RPI * j + fill_row;
+    const int chunk = fill_pos ^ lds_swz<D>(row);
+    koff[j] = (uint32_t)((row * ks2 + chunk * 8) * (int64_t)sizeof(T));
+    voff[j] = (uint32_t)((row * vs2 + chunk * 8) * (int64_t)sizeof(T));
   }
-  auto load_tile = [&](int kv0_in) {
+  auto issue_tile = [&](auto stage, int kv0_in) {
+    T* const Kst = stage_ptr(stage, Ksm0, Ksm1);
+    T* const Vst = stage_ptr(stage, Vsm0, Vsm1);
     const int kv0 = __builtin_amdgcn_readfirstlane(kv0_in);
-    if (kv0 + BN <= p.Lkv) {
-      const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)kv0 * ks2);
-      const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)kv0 * vs2);
+    const int lim = p.Lkv - 1 - kv0;
+    const int r0 = 16 * wu;
+    if (lim >= BN - 1) {
+      const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)(kv0 + r0) * ks2);
+      const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)(kv0 + r0) * vs2);
 #pragma unroll
-      for (int j = 0; j < NLD; j++) {
-        kreg[j] = *reinterpret_cast<const u32x4*>(kt + klo[j]);
-        if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vt + vlo[j]);
+      for (int j = 0; j < NI; j++) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt + koff[j]),
+                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * j) * D), 16, 0, 0);
+        if constexpr (PASS != kFwdLse)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt + voff[j]),
+                                           (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * j) * D), 16, 0, 0);
       }
     } else {
+      // the last tile of a ragged length: rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
-      for (int j = 0; j < NLD; j++) {
-        const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-        const int kvc = min(kv0 + r, p.Lkv - 1);  // rows past the end: clamped (finite filler, masked out below)
-        kreg[j] = *reinterpret_cast<const u32x4*>(kbase + (int64_t)kvc * ks2 + cc * 8);
-        if constexpr (PASS != kFwdLse) vreg[j] = *reinterpret_cast<const u32x4*>(vbase + (int64_t)kvc * vs2 + cc * 8);
+      for (int j = 0; j < NI; j++) {
+        const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);
+        const int row = min(r0 + RPI * j + fill_row, lim);
+        const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
+        const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
+                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * j) * D), 16, 0, 0);
+        if constexpr (PASS != kFwdLse)
+          __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
+                                           (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * j) * D), 16, 0, 0);
       }
     }
   };
-  auto store_tile = [&](int stage) {
+  // element offsets inside a 32-row block: row fragments (row i32, chunk 2s + g sits at (2s) ^ kz) and
+  // transposing reads (4 elements of row 4g + (i16 >> 2) + 8e, logical column 32db + 16hh + 4(i16 & 3))
+  const int kz = g ^ lds_swz<D>(i32);
+  int toff[2][DB];
+  {
+    const int rl = 4 * g + (i16 >> 2), hh = (lane >> 4) & 1;
 #pragma unroll
-    for (int j = 0; j < NLD; j++) {
-      const int c = tid + 256 * j, r = c / CPR, cc = c % CPR;
-      *reinterpret_cast<u32x4*>(Ksm[stage] + r * ROWE + cc * 8) = kreg[j];
-      if constexpr (PASS != kFwdLse) *reinterpret_cast<u32x4*>(Vsm[stage] + r * ROWE + cc * 8) = vreg[j];
-    }
-  };
+    for (int e = 0; e < 2; e++)
+#pragma unroll
+      for (int db = 0; db < DB; db++) {
+        const int chunk = 4 * db + 2 * hh + ((i16 & 3) >> 1);
+        toff[e][db] = (rl + 8 * e) * D + ((chunk ^ lds_swz<D>(rl + 8 * e)) * 8) + 4 * (i16 & 1);
+      }
+  }
 
   Score2<KIND> sm;
   sm.init(p.score, p.scale, h, b, p.Lq, p.Lkv);
@@ -184,27 +213,23 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
   constexpr float kPGuard = 32768.f, kPTiny = 1.f / 64.f;
   int t_cur = it0 < it1 ? tile_at(it0) : 0;
   int t_nxt = it0 + 1 < it1 ? tile_at(it0 + 1) : 0;
-  // prologue: the first tile into its stage, the second into registers
-  int any_tile = it0 < it1;
-  if (any_tile) load_tile(t_cur * BN);
-  // Unconditional, and as an instruction the compiler's wait-count pass sees: the Q fragments (and tile 0) have
-  // arrived.  With the wait only inside the branch the pass carries "Q fragments may still be in flight" into
-  // the loop and makes the first products of every tile wait for all outstanding loads, i.e. for the prefetch of the
-  // tile after next that was issued half a tile earlier.  The condition is made opaque in between so that the two
-  // branches around the wait are not merged into one (which moves a copy of the wait into each arm).
-  asm volatile("" : "+v"(any_tile));
-  any_tile = __builtin_amdgcn_readfirstlane(any_tile);
-  __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-  if (any_tile) store_tile(it0 & 1);
-  if (it0 + 1 < it1) load_tile(t_nxt * BN);
+  if (it0 < it1) issue_tile(StageC<0>{}, t_cur * BN);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the Q fragments and this wave's share of the first tile
   __syncthreads();
-  for (int it = it0; it < it1; it++) {
+  // one tile out of the stage named by `stage` (= (it - it0) & 1)
+  auto tile_step = [&](auto stage, int it) {
+    constexpr int ST = decltype(stage)::value;
     const int kv0 = t_cur * BN;
     const bool masked = (it < n_part) || (kv0 + BN > p.Lkv);
-    const T* Ks = Ksm[it & 1];
-    const T* Vs = Vsm[PASS == kFwdLse ? 0 : (it & 1)];
-    t_cur = t_nxt;
-    if (it + 2 < it1) t_nxt = tile_at(it + 2);
+    const T* const Ks = stage_ptr(stage, Ksm0, Ksm1);
+    const T* const Vs = stage_ptr(stage, Vsm0, Vsm1);
+    if (it + 1 < it1) {
+      // the other stage was last read before the previous barrier: the next tile lands there while this one is
+      // consumed; the tile index after that is looked up a tile ahead
+      issue_tile(StageC<1 - ST>{}, t_nxt * BN);
+      t_cur = t_nxt;
+      if (it + 2 < it1) t_nxt = tile_at(it + 2);
+    }
 
     // Each 32-row half of the tile is one online-softmax step.
 #pragma unroll
@@ -225,16 +250,16 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
       // ---- operand fragments of this step: K rows, and V columns (transposed reads) ----
       vec8 kfr[DS], vfr[2][DB];
       {
-        const T* kp = Ks + (nb * 32 + i32) * ROWE + 8 * g;
+        const T* kp = Ks + (nb * 32 + i32) * D;
 #pragma unroll
-        for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + 16 * s);
+        for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + (((2 * s) ^ kz) * 8));
         if constexpr (PASS != kFwdLse) {
 #pragma unroll
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
             for (int db = 0; db < DB; db++) {
-              const T* vp = Vs + (32 * nb + 16 * tt + 4 * g + (i16 >> 2)) * ROWE + 32 * db + 16 * ((lane >> 4) & 1) + 4 * (i16 & 3);
-              vfr[tt][db] = join8<vec8>(lds_read_tr(vp), lds_read_tr(vp + 8 * ROWE));
+              const T* vp = Vs + (32 * nb + 16 * tt) * D;
+              vfr[tt][db] = join8<vec8>(lds_read_tr(vp + toff[0][db]), lds_read_tr(vp + toff[1][db]));
             }
         }
       }
@@ -351,14 +376,14 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, cons
         }
       }
       }  // block not entirely hidden
-      if (nb == 0 && it + 1 < it1) {
-        // the other stage was last read before the previous barrier: refill it with the
-        // tile prefetched into registers, then start fetching the one after
-        store_tile((it + 1) & 1);
-        if (it + 2 < it1) load_tile(t_nxt * BN);
-      }
     }
+    // this wave's share of the next tile has landed; after the barrier everyone's has
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+  };
+  for (int it = it0; it < it1; it += 2) {
+    tile_step(StageC<0>{}, it);
+    if (it + 1 < it1) tile_step(StageC<1>{}, it + 1);
   }
 
   // ---- epilogue ----
