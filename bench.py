@@ -49,9 +49,9 @@ PEAK_HBM_GBPS = 8000.0
 # Keyed by (workload, kernel); a kernel that has not been measured reports null.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_config2_and_decode_pmc.md"
 MEASURED_TRAFFIC_BYTES = {
-    ("config2", "fwd_pipe_kernel"): 67977441,
-    ("config2", "bwd_dq_kernel"): 136135883,
-    ("config2", "bwd_dkv_kernel"): 137466890,
+    ("config2", "fwd_pipe_kernel"): 67954311,
+    ("config2", "bwd_dq_kernel"): 136180161,
+    ("config2", "bwd_dkv_kernel"): 137453189,
 }
 
 
