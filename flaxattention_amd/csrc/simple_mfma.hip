@@ -52,7 +52,7 @@ static int dispatch(const FlexAttnParams& p, const SimpleArgs& a) {
 // workgroup per compute unit, with at least 16 steps of 32 keys each.
 int flex_simple_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kSimpleQTile - 1) / kSimpleQTile) * p.Hq * p.B;
-  if (wgs >= 128) return 1;
+  if (wgs > 128) return 1;
   const int steps = (p.Lkv + kSimpleStep - 1) / kSimpleStep;
   int s = (int)(256 / wgs);
   if (s > steps / 16) s = steps / 16;
