@@ -283,7 +283,7 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
         else:
             # few query tiles against many keys: with a workspace the library may split the call over the keys
             ws = None
-            if plan.split_kv and plan.B * plan.Hq * ((plan.Lq + 127) // 128) < 256 and plan.Lkv >= 1024:
+            if plan.split_kv and plan.B * plan.Hq * ((plan.Lq + 127) // 128) <= 256 and plan.Lkv >= 1024:
                 nbytes = L.flexattn_fwd_workspace_bytes(p)
                 if nbytes:
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)

@@ -39,11 +39,12 @@ bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
 }
 
 // Shares of the key tiles a forward call is split into (1 = none): calls whose query tiles alone would leave most
-// compute units without a workgroup (fewer than one per compute unit) -- few rows against a long key sequence -- are
-// split until there are about two workgroups per compute unit, with at least 8 tiles of 64 keys each.
+// compute units without a workgroup, or with one where two fit (at most one per compute unit) -- few rows against a
+// long key sequence -- are split until there are about two workgroups per compute unit, with at least 8 tiles of 64
+// keys each.
 int flex_mfma_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B;
-  if (wgs >= 256) return 1;
+  if (wgs > 256) return 1;
   const int tiles = (p.Lkv + kFwdBN - 1) / kFwdBN;
   int s = (int)(512 / wgs);
   if (s > tiles / 8) s = tiles / 8;
