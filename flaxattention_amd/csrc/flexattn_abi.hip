@@ -126,8 +126,8 @@ extern "C" size_t flexattn_fwd_workspace_bytes(const FlexAttnParams* p) {
   size_t n = fwd_lse_bytes(p);
   // the matrix-core forward kernels split the keys of a call with few query tiles over several workgroups, whose
   // partial results live here
-  if (wants_fused(p) && flex_simple_supported(*p, 0)) n += flex_simple_fwd_partial_bytes(*p, flex_simple_fwd_splits(*p));
-  else if (wants_fused(p) && flex_mfma_fwd_supported(*p)) n += flex_mfma_fwd_partial_bytes(*p, flex_mfma_fwd_splits(*p));
+  if (wants_fused(p) && flex_mfma_fwd_supported(*p)) n += flex_mfma_fwd_partial_bytes(*p, flex_mfma_fwd_splits(*p));
+  else if (wants_fused(p) && flex_simple_supported(*p, 0)) n += flex_simple_fwd_partial_bytes(*p, flex_simple_fwd_splits(*p));
   return n;
 }
 
@@ -140,7 +140,7 @@ extern "C" int flexattn_fwd(const FlexAttnParams* p, const void* q, const void* 
   int rc;
   // the simple matrix-core kernels: float32 inputs (the reference rounds nothing below fp32, so every numerics mode
   // but FLEX_STRICT is the same computation) and the 16-bit head sizes above 128
-  if (wants_fused(p) && flex_simple_supported(*p, 0)) {
+  if (wants_fused(p) && flex_simple_supported(*p, 0) && !flex_mfma_fwd_supported(*p)) {
     const FlexAttnParams ps = with_parity_resolved(p, true);
     if ((ps.flags & FLEX_PARITY) && p->dtype != FLEX_F32 && !lse2) {
       if (!workspace) { flex_set_error("flexattn_fwd: FLEX_PARITY needs lse2 or a workspace of flexattn_fwd_workspace_bytes()"); return 1; }

@@ -1,4 +1,4 @@
-// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128}).
+// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128}; the list-driven kernel also 256).
 //
 // Takes the place of mha_forward_kernel (flaxattention/kernel/attention.py:
 // 34-149) and of the dense math path (flaxattention/core/attention.py:14-106)
@@ -42,8 +42,10 @@ constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dens
 //                instructions per fragment) and the row sum adds the unrounded exponentials: the "unrounded"
 //                numerics, launched with ROUND_S = false
 enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2, kFwdHiLo = 3 };
+// D = 256: one wave per SIMD (Q fragments, K / V fragments and the accumulator are 64 + 128 + 128 registers; the
+// one-pass instantiations spill about 50 more, the two passes of the parity numerics none) and the two stages are 128 KB.
 template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
-__global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2,
                                                            float* __restrict__ o_part, float* __restrict__ ml_part) {

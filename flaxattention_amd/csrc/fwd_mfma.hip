@@ -1,4 +1,4 @@
-// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128}): checks and dispatch.  The kernels
+// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128, 256}): checks and dispatch.  The kernels
 // are in fwd_mfma.cuh, instantiated per (dtype, head size) by fwd_mfma_inst.hip.
 #include "fwd_mfma.cuh"
 
@@ -8,6 +8,8 @@ int flex_mfma_fwd_f16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_f16_128(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_128(const FlexAttnParams& p, const FwdArgs& a);
+int flex_mfma_fwd_f16_256(const FlexAttnParams& p, const FwdArgs& a);
+int flex_mfma_fwd_bf16_256(const FlexAttnParams& p, const FwdArgs& a);
 
 // rows of 16-byte chunks; the kernels keep the offset of a row inside a tile in 32 bits
 static bool strides_ok(const int64_t* s) { return s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && s[2] >= 0 && s[2] < (1 << 24); }
@@ -33,7 +35,15 @@ void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
 }
 
 bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
-  if (!flex_mfma_shape_ok(p)) return false;
+  if (p.D == 256 && p.Dv == 256) {
+    // the list-driven forward is also instantiated for 256-wide heads (one wave per SIMD); everything but the head
+    // size is checked as for 128
+    FlexAttnParams as128 = p;
+    as128.D = as128.Dv = 128;
+    if (!flex_mfma_shape_ok(as128)) return false;
+  } else if (!flex_mfma_shape_ok(p)) {
+    return false;
+  }
   const FlexTileLists& t = p.tiles;
   return !t.kv_num || (t.q_block == kFwdBM && t.kv_block == kFwdBN);
 }
@@ -44,9 +54,10 @@ bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
 // keys each.
 int flex_mfma_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B;
-  if (wgs > 256) return 1;
+  const int slots = p.D == 256 ? 256 : 512;  // 256-wide heads run one workgroup per compute unit
+  if (wgs > slots / 2) return 1;
   const int tiles = (p.Lkv + kFwdBN - 1) / kFwdBN;
-  int s = (int)(512 / wgs);
+  int s = (int)(slots / wgs);
   if (s > tiles / 8) s = tiles / 8;
   if (s > 64) s = 64;  // the merge kernel takes one split per lane
   return s < 2 ? 1 : s;
@@ -79,8 +90,8 @@ int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const v
     a.ml_part = a.o_part + (size_t)p.B * p.Hq * p.Lq * splits * p.D;
   }
   int rc = 1;
-  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_mfma_fwd_f16_64(p, a) : flex_mfma_fwd_f16_128(p, a);
-  else rc = p.D == 64 ? flex_mfma_fwd_bf16_64(p, a) : flex_mfma_fwd_bf16_128(p, a);
+  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_mfma_fwd_f16_64(p, a) : p.D == 128 ? flex_mfma_fwd_f16_128(p, a) : flex_mfma_fwd_f16_256(p, a);
+  else rc = p.D == 64 ? flex_mfma_fwd_bf16_64(p, a) : p.D == 128 ? flex_mfma_fwd_bf16_128(p, a) : flex_mfma_fwd_bf16_256(p, a);
   if (rc) flex_set_error("fused forward: unsupported score_mod kind %d", p.score.kind);
   return rc;
 }
