@@ -42,14 +42,14 @@ constexpr int kListBN = 128; // key granularity of the backward tile lists = key
 //                as a high and a low part (two matrix instructions per fragment); launched with ROUND_S = false
 enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2, kBwdDeltaRaw = 3, kBwdHiLo = 4 };
 // keys the dQ kernel stages per step (the kernel and the launcher that picks its mask-free instantiation agree on it)
-template <int D, int MODE> constexpr int dq_tile_keys() { return (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2; }
+template <int D, int MODE> constexpr int dq_tile_keys() { return D == 256 ? kBN / 2 : (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2; }
 // Registers: two waves per SIMD (256 registers each) everywhere but the fast-numerics kernel at D = 128, which then
 // spills 31 - 59 registers and reloads them inside the tile loop (every reload is a vector memory load, and a wait for
 // one is a wait for the tile fetch in flight as well); with one wave per SIMD and no spill it is 10 - 15 % faster
 // ([4,16,4096,128] bf16: 1213 -> 1031 us dense, 603 -> 544 us causal).  The row sweep does not spill; the parity kernel
 // (19 - 52 registers spilled) loses 22 % with one wave per SIMD and the high/low kernel gains nothing, so they keep two.
 template <typename T, int D, int KIND, bool ROUND_S, bool MASKED, int MODE = kBwdFast>
-__global__ __launch_bounds__(256, (D == 128 && MODE == kBwdFast) ? 1 : 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D == 256) ? 1 : 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
                                                       const T* __restrict__ d_o, T* __restrict__ dq,
@@ -698,8 +698,13 @@ struct BwdArgs {
   hipStream_t s;
 };
 
+// (D = 256 has the dQ kernel only: the resident K / V fragments and the two accumulators of a dK/dV workgroup do not
+// fit a wave's registers; the caller runs the dK/dV kernel of the simple family)
 template <typename T, int D, int KIND, bool RS, bool BITS, bool PARITY, bool HILO = false>
 static int launch_dkv_as(const FlexAttnParams& p, const BwdArgs& a) {
+  if constexpr (D == 256) {
+    return 3;
+  } else {
   constexpr size_t sm = dkv_smem<D, T>();
   // set on every call: the attribute is per device, and a remembered "already set" would be neither
   // per device nor safe between threads (the call is a host-side table update, no device work)
@@ -710,6 +715,7 @@ static int launch_dkv_as(const FlexAttnParams& p, const BwdArgs& a) {
   hipLaunchKernelGGL((bwd_dkv_kernel<T, D, KIND, RS, BITS, PARITY, HILO>), dim3(nkt * p.Hkv * p.B), dim3(DkvShape<D>::kThreads), sm, a.s,
                      p, (const T*)a.q, (const T*)a.k, (const T*)a.v, a.lse2, a.delta, (const T*)a.d_o, (T*)a.dk, (T*)a.dv);
   return 0;
+  }
 }
 template <typename T, int D, int KIND, bool RS, bool PARITY>
 static int launch_dkv(const FlexAttnParams& p, const BwdArgs& a) {
@@ -727,8 +733,13 @@ static void launch_dq_as(const FlexAttnParams& p, const BwdArgs& a) {
 template <typename T, int D, int KIND, bool RS>
 static void launch_dq(const FlexAttnParams& p, const BwdArgs& a) {
   constexpr int BN = dq_tile_keys<D, kBwdFast>();   // the kernel's key tile
-  if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0) launch_dq_as<T, D, KIND, RS, false, kBwdFast>(p, a);
-  else launch_dq_as<T, D, KIND, RS, true, kBwdFast>(p, a);
+  if constexpr (D != 256) {  // (at D = 256 the mask-free instantiation is the one that spills: not used)
+    if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0) {
+      launch_dq_as<T, D, KIND, RS, false, kBwdFast>(p, a);
+      return;
+    }
+  }
+  launch_dq_as<T, D, KIND, RS, true, kBwdFast>(p, a);
 }
 
 template <typename T, int D, int KIND, bool RS>

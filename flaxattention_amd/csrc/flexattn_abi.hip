@@ -23,6 +23,7 @@ size_t flex_mfma_fwd_partial_bytes(const FlexAttnParams& p, int splits);
 int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
                   void* partials, hipStream_t s);
 bool flex_mfma_bwd_supported(const FlexAttnParams& p);
+bool flex_mfma_dq256_supported(const FlexAttnParams& p);
 size_t flex_mfma_bwd_workspace(const FlexAttnParams& p);
 int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                   const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
@@ -188,7 +189,15 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
   hipStream_t s = (hipStream_t)stream;
   int rc;
   if (wants_fused(p) && flex_simple_supported(*p, 1)) {
-    const FlexAttnParams ps = with_parity_resolved(p, true);
+    FlexAttnParams ps = with_parity_resolved(p, true);
+    if (flex_mfma_dq256_supported(ps) && !(ps.flags & (FLEX_BWD_ONLY_DQ | FLEX_BWD_ONLY_DKV))) {
+      // 256-wide heads: dQ (and the row sweep for delta, which the dK/dV kernel reads from the workspace) on the tuned
+      // kernel, dK/dV on the simple one
+      FlexAttnParams pq = ps;
+      pq.flags |= FLEX_BWD_ONLY_DQ;
+      if (int rcq = flex_mfma_bwd(pq, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s)) return rcq;
+      ps.flags |= FLEX_BWD_ONLY_DKV;
+    }
     if (int rcs = flex_simple_bwd(ps, q, k, v, o, lse2, d_o, dq, dk, dv, workspace, s)) return rcs;
     return check_launch("flexattn_bwd");
   }
