@@ -42,8 +42,8 @@ constexpr int kPipeBM = 256;  // query rows of a workgroup of the pipelined dens
 //                instructions per fragment) and the row sum adds the unrounded exponentials: the "unrounded"
 //                numerics, launched with ROUND_S = false
 enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2, kFwdHiLo = 3 };
-// D = 256: one wave per SIMD (Q fragments, K / V fragments and the accumulator are 64 + 128 + 128 registers; the
-// one-pass instantiations spill about 50 more, the two passes of the parity numerics none) and the two stages are 128 KB.
+// D = 256: one wave per SIMD (Q fragments, K fragments and the accumulator are 64 + 64 + 128 registers, the V
+// fragments another 64 that are fetched late) and the two stages are 128 KB.
 template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
 __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
@@ -255,7 +255,9 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
         const T* kp = Ks + (nb * 32 + i32) * D;
 #pragma unroll
         for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + (((2 * s) ^ kz) * 8));
-        if constexpr (PASS != kFwdLse) {
+        // (D = 256: the 64 registers of V fragments are fetched right before their product instead, or the block
+        // would not fit a wave's registers)
+        if constexpr (PASS != kFwdLse && D != 256) {
 #pragma unroll
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
@@ -372,6 +374,10 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
             for (int db = 0; db < DB; db++) {
+              if constexpr (D == 256) {
+                const T* vp = Vs + (32 * nb + 16 * tt) * D;
+                vfr[tt][db] = join8<vec8>(lds_read_tr(vp + toff[0][db]), lds_read_tr(vp + toff[1][db]));
+              }
               oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf[tt], oacc[a][db]);
               if constexpr (PASS == kFwdHiLo) oacc[a][db] = Frag<T>::mfma(vfr[tt][db], pf_lo[tt], oacc[a][db]);
             }
