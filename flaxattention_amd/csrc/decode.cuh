@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (
   // V strips: per wave NSTG stages of 32 unpadded swizzled rows, filled global -> LDS directly (no staging
   // registers).  The same memory serves the cross-wave reduction of the partial outputs at the end.
   // NSTG V strips per wave and DEPTH = NSTG - 1 steps of loads in flight while one is computed.  Three strips and two
-  // sets of K registers (two steps ahead) were measured at D = 64 and change nothing (config 5, one workgroup per
+  // sets of K registers (two steps ahead) were measured at D = 64 and change nothing (fp16 KV cache [8,8,16384,64], one workgroup per
   // compute unit: 53.2 us against 52.9 us at q_len 1, 57.1 against 55.7 at q_len 64): the bytes in flight are not what
   // limits this kernel, so two strips and one step ahead it stays.
   constexpr int NSTG = 2, DEPTH = NSTG - 1;

@@ -53,7 +53,7 @@ bool flex_decode_supported(const FlexAttnParams& p) {
 
 int flex_decode_default_splits(const FlexAttnParams& p) {
   // ONE workgroup per compute unit: a bandwidth-bound kernel gains nothing from more, and every further split adds
-  // partials to write and merge (config 5 at q_len 1: 53 us with 4 splits = 256 workgroups, 54 us with 8, 58 us with
+  // partials to write and merge (fp16 KV cache [8,8,16384,64] at q_len 1: 53 us with 4 splits = 256 workgroups, 54 us with 8, 58 us with
   // 16; at q_len 64: 56 us with 4, 60 us with 8).  At least 8 steps each.
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
