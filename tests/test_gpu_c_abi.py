@@ -139,3 +139,64 @@ def test_decode_with_lists_of_another_granularity(dev):
     want = fa.flax_attention(q, k, v, block_mask=fa.create_block_mask(spec_off, 1, 1, Lq, Lkv, device=dev),
                              kernel_options={"decode": False})
     assert max_abs(outs[0].cpu(), want.cpu()) <= 4e-3
+
+
+def test_threads_on_their_own_streams(dev):
+    """The entry points keep no state between calls: two host threads, each on a stream of its own, run forward +
+    backward (tuned, simple and decode kernels) on different problems at the same time; every result equals, bit for
+    bit, the one of the same call made alone.  An error in one thread leaves the other thread's error string alone."""
+    import threading
+    import flaxattention_amd as fa
+    from flaxattention_amd.masks import causal_mask
+    from flaxattention_amd.mods import generate_alibi_bias
+    torch.cuda.synchronize()
+    cases = [(torch.float16, 2, 4, 384, 384, 64), (torch.bfloat16, 1, 4, 300, 520, 128),
+             (torch.float32, 1, 2, 256, 256, 64), (torch.float16, 2, 4, 8, 2048, 128)]
+
+    def work(seed, out):
+        res = []
+        for i, (dtype, B, H, Lq, Lkv, D) in enumerate(cases):
+            g = torch.Generator(device=dev).manual_seed(100 * seed + i)
+            q, k, v = (torch.randn(B, H, L, D, generator=g, device=dev, dtype=torch.float32).to(dtype).requires_grad_(True)
+                       for L in (Lq, Lkv, Lkv))
+            bm = fa.create_block_mask(causal_mask, 1, 1, Lq, Lkv, device=dev) if Lq == Lkv else None
+            o, lse = fa.flax_attention(q, k, v, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, return_lse=True)
+            grads = torch.autograd.grad(o.float().square().sum(), (q, k, v))
+            res.append((o.detach(), lse.detach()) + tuple(grads))
+        out[seed] = res
+
+    alone = {}
+    for seed in (1, 2):
+        work(seed, alone)
+    torch.cuda.synchronize()
+    together, errors = {}, {}
+
+    def threaded(seed):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream(device=dev)):
+                for _ in range(3):
+                    work(seed, together)
+                if seed == 2:   # an error of this thread's own
+                    L = _lib.lib()
+                    q, k, v = _inputs(dev, 1, 2, 128, 128, 64)
+                    p = _params(q, k, v, torch.empty_like(q))
+                    assert L.flexattn_fwd(p, None, k.data_ptr(), v.data_ptr(), q.data_ptr(), None, None, _stream()) != 0
+                    errors[seed] = L.flexattn_last_error()
+                else:
+                    errors[seed] = _lib.lib().flexattn_last_error()
+                torch.cuda.current_stream().synchronize()
+        except Exception as e:   # pragma: no cover
+            errors[seed] = e
+
+    threads = [threading.Thread(target=threaded, args=(s,)) for s in (1, 2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert isinstance(errors[2], bytes) and b"null" in errors[2], errors[2]
+    assert isinstance(errors[1], bytes) and b"null" not in errors[1], errors[1]
+    for seed in (1, 2):
+        for a, b in zip(alone[seed], together[seed]):
+            for x, y in zip(a, b):
+                assert torch.equal(x, y)
