@@ -37,8 +37,8 @@ selects numerics here:
     {"backend": "generic" | "auto"}
     {"decode": bool}      split-KV decode kernel on / off; by default it is used
                           whenever it applies (fp16/bf16, D = Dv in {64, 128} with
-                          at most 64 query rows per KV head or D = Dv = 256 with at
-                          most 32, at least 512 keys); True also runs longer queries
+                          at most 64 query rows per KV head or D = Dv in {192, 256}
+                          with at most 32, at least 512 keys); True also runs longer queries
                           through it, in chunks of that many rows
     {"decode_splits": n}  force the split-KV decode kernel with n splits
     {"split_kv": bool}    False: the forward kernel never splits a call over the keys
@@ -210,7 +210,7 @@ def _decode_choice(q, k, v, score: ScoreMod, flags: int, opts: dict) -> int:
         return 0
     B, Hq, Lq, D = q.shape
     G = Hq // k.shape[1]
-    ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128, 256)
+    ok = (q.dtype in (torch.float16, torch.bfloat16) and D == v.shape[3] and D in (64, 128, 192, 256)
           and score.kind != _lib.SCORE_AFFINE
           and not (flags & (_lib.FLAG_STRICT | _lib.FLAG_FORCE_GENERIC | _lib.FLAG_UNROUNDED)))
     if want is True:

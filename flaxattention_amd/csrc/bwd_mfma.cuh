@@ -42,14 +42,14 @@ constexpr int kListBN = 128; // key granularity of the backward tile lists = key
 //                as a high and a low part (two matrix instructions per fragment); launched with ROUND_S = false
 enum { kBwdFast = 0, kBwdDelta = 1, kBwdParity = 2, kBwdDeltaRaw = 3, kBwdHiLo = 4 };
 // keys the dQ kernel stages per step (the kernel and the launcher that picks its mask-free instantiation agree on it)
-template <int D, int MODE> constexpr int dq_tile_keys() { return D == 256 ? kBN / 2 : (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2; }
+template <int D, int MODE> constexpr int dq_tile_keys() { return D >= 192 ? kBN / 2 : (D == 64 || MODE == kBwdFast) ? kBN : kBN / 2; }
 // Registers: two waves per SIMD (256 registers each) everywhere but the fast-numerics kernel at D = 128, which then
 // spills 31 - 59 registers and reloads them inside the tile loop (every reload is a vector memory load, and a wait for
 // one is a wait for the tile fetch in flight as well); with one wave per SIMD and no spill it is 10 - 15 % faster
 // ([4,16,4096,128] bf16: 1213 -> 1031 us dense, 603 -> 544 us causal).  The row sweep does not spill; the parity kernel
 // (19 - 52 registers spilled) loses 22 % with one wave per SIMD and the high/low kernel gains nothing, so they keep two.
 template <typename T, int D, int KIND, bool ROUND_S, bool MASKED, int MODE = kBwdFast>
-__global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D == 256) ? 1 : 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D >= 192) ? 1 : 2) void bwd_dq_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                       const T* __restrict__ k, const T* __restrict__ v,
                                                       const T* __restrict__ o, const float* __restrict__ lse2,
                                                       const T* __restrict__ d_o, T* __restrict__ dq,
@@ -60,8 +60,10 @@ __global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D == 256) ?
   // D = 128 runs one wave per SIMD (see above), has the 128 KB for 128-key tiles and is 3 - 6 % faster with them
   constexpr int BM = kBM, BN = dq_tile_keys<D, MODE>();
   constexpr int DS = D / 16, DB = D / 32, CPR = D / 8;
-  constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
-  constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor
+  // a wave fills BN / 4 rows of a tile: (BN / 4) * CPR chunks, 64 per fetch instruction, laid down one after the
+  // other (at D = 192 an instruction ends in the middle of a row); the fetch pattern repeats every 16 rows
+  constexpr int NI = (BN / 4) * CPR / 64;   // fetch instructions per wave, tile and tensor
+  static_assert(((BN / 4) * CPR) % 64 == 0 && (16 * CPR) % 64 == 0, "whole fetch instructions per swizzle period");
   // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled
   // rows): while one tile is consumed the next one lands, one workgroup barrier per tile.  Each stage is a
   // variable of its own and every access names its stage at compile time (the tile loop is unrolled by two):
@@ -142,16 +144,15 @@ __global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D == 256) ?
   const int64_t ks2 = p.k_stride[2], vs2 = p.v_stride[2];
   // tile fetch: wave w fills rows [32w, 32w + 32) of the K and the V tile, RPI rows per instruction;
   // the lane that fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row
-  const int fill_row = lane / CPR, fill_pos = lane % CPR;
   // the per-lane part of a fetch address (row among the 16 of a swizzle period, swizzled chunk) is the same for
   // every tile: kept as byte offsets from a wave-uniform row address
   const int wu = __builtin_amdgcn_readfirstlane(w);
-  constexpr int NP = 16 / RPI;  // fetch instructions per swizzle period
+  constexpr int NP = 16 * CPR / 64;  // fetch instructions per swizzle period
   uint32_t koff[NP], voff[NP];
 #pragma unroll
   for (int jp = 0; jp < NP; jp++) {
-    const int row = RPI * jp + fill_row;
-    const int chunk = fill_pos ^ lds_swz<D>(row);  // the wave's first row is a multiple of 16
+    const int c = 64 * jp + lane, row = c / CPR;
+    const int chunk = (c % CPR) ^ lds_swz<D>(row);  // the wave's first row is a multiple of 16
     koff[jp] = (uint32_t)((row * ks2 + chunk * 8) * (int64_t)sizeof(T));
     voff[jp] = (uint32_t)((row * vs2 + chunk * 8) * (int64_t)sizeof(T));
   }
@@ -163,27 +164,27 @@ __global__ __launch_bounds__(256, ((D == 128 && MODE == kBwdFast) || D == 256) ?
     if (lim >= BN - 1) {
 #pragma unroll
       for (int j = 0; j < NI; j++) {
-        const int r0 = (BN / 4) * wu + RPI * (j - j % NP);
+        const int r0 = (BN / 4) * wu + 16 * (j / NP);   // first row of the swizzle period instruction j belongs to
         const char* kt = reinterpret_cast<const char*>(kbase + (int64_t)(kv0 + r0) * ks2);
         const char* vt = reinterpret_cast<const char*>(vbase + (int64_t)(kv0 + r0) * vs2);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt + koff[j % NP]),
-                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * (j % NP)) * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D + 512 * (j % NP)), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt + voff[j % NP]),
-                                         (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * (j % NP)) * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Vst + r0 * D + 512 * (j % NP)), 16, 0, 0);
       }
     } else {
       // the last tile of a ragged length: rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
       for (int j = 0; j < NI; j++) {
-        const int r0 = (BN / 4) * wu + RPI * j;
-        const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);
-        const int row = min(r0 + fill_row, lim);
+        const int c = 64 * j + lane, rw = c / CPR;      // row inside the wave's share, and its chunk position
+        const int chunk = (c % CPR) ^ lds_swz<D>(rw);
+        const int row = min((BN / 4) * wu + rw, lim);
         const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
         const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
-                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Kst + (BN / 4) * wu * D + 512 * j), 16, 0, 0);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                         (__attribute__((address_space(3))) void*)(Vst + r0 * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Vst + (BN / 4) * wu * D + 512 * j), 16, 0, 0);
       }
     }
   };
@@ -698,11 +699,11 @@ struct BwdArgs {
   hipStream_t s;
 };
 
-// (D = 256 has the dQ kernel only: the resident K / V fragments and the two accumulators of a dK/dV workgroup do not
+// (D = 192 and D = 256 have the dQ kernel only: the resident K / V fragments and the two accumulators of a dK/dV workgroup do not
 // fit a wave's registers; the caller runs the dK/dV kernel of the simple family)
 template <typename T, int D, int KIND, bool RS, bool BITS, bool PARITY, bool HILO = false>
 static int launch_dkv_as(const FlexAttnParams& p, const BwdArgs& a) {
-  if constexpr (D == 256) {
+  if constexpr (D >= 192) {
     return 3;
   } else {
   constexpr size_t sm = dkv_smem<D, T>();
@@ -733,7 +734,7 @@ static void launch_dq_as(const FlexAttnParams& p, const BwdArgs& a) {
 template <typename T, int D, int KIND, bool RS>
 static void launch_dq(const FlexAttnParams& p, const BwdArgs& a) {
   constexpr int BN = dq_tile_keys<D, kBwdFast>();   // the kernel's key tile
-  if constexpr (D != 256) {  // (at D = 256 the mask-free instantiation is the one that spills: not used)
+  if constexpr (D < 192) {  // (at D = 192 / 256 the mask-free instantiation is the one that spills: not used)
     if (!p.tiles_bwd.kv_num && mask_hides_nothing(p.mask) && p.Lkv % BN == 0) {
       launch_dq_as<T, D, KIND, RS, false, kBwdFast>(p, a);
       return;

@@ -16,17 +16,20 @@ constexpr int kStep = 32;  // KV rows per wave step
 //                kernel sums them)
 enum { kDecOnePass = 0, kDecLse = 1, kDecNorm = 2 };
 template <typename T, int D, int KIND, bool ROUND_S, int NB, int PASS = kDecOnePass>
-__global__ __launch_bounds__(256, D == 256 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D >= 192 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (D == 64 ? 2 : 1)) void decode_split_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                             const T* __restrict__ k, const T* __restrict__ v,
                                                             float* __restrict__ o_part, float* __restrict__ ml_part,
                                                             int splits, const float* __restrict__ lse_in) {
   typedef typename Frag<T>::vec8 vec8;
   // D = 256 serves one column block: the two V strips of the four waves are 128 KB of the 160 KB of LDS, which leaves
-  // no room for a second block's Q fragments, and its registers (64 for Q, 64 for K, 128 for O) no room to keep them
-  static_assert(D == 64 || D == 128 || (D == 256 && NB == 1), "decode_split_kernel: head size / column blocks");
+  // no room for a second block's Q fragments, and its registers (64 for Q, 64 for K, 128 for O) no room to keep them;
+  // D = 192 likewise runs one wave per SIMD with one column block
+  static_assert(D == 64 || D == 128 || ((D == 192 || D == 256) && NB == 1), "decode_split_kernel: head size / column blocks");
   constexpr int DS = D / 16, DB = D / 32, ROWE = D + 8, CPR = D / 8;
-  constexpr int RPI = 64 / CPR;        // V rows one wave-wide fetch instruction fills
-  constexpr int NVI = kStep / RPI;     // fetch instructions per step
+  // a strip is kStep * CPR chunks, 64 per wave-wide fetch instruction, laid down one after the other (at D = 192 an
+  // instruction ends in the middle of a row)
+  constexpr int NVI = kStep * CPR / 64;  // fetch instructions per step
+  static_assert((kStep * CPR) % 64 == 0, "whole fetch instructions per strip");
   // V strips: per wave NSTG stages of 32 unpadded swizzled rows, filled global -> LDS directly (no staging
   // registers).  The same memory serves the cross-wave reduction of the partial outputs at the end.
   // NSTG V strips per wave and DEPTH = NSTG - 1 steps of loads in flight while one is computed.  Three strips and two
@@ -123,7 +126,6 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (
   const int last = p.Lkv - 1;
   vec8 kfA[DS], kfB[DS];  // two sets of K registers, named so that they stay in registers (kfB unused at DEPTH 1)
   T* Vw = reinterpret_cast<T*>(vs_red) + w * NSTG * kStripElems;
-  const int fill_row = lane / CPR, fill_pos = lane % CPR;
   // V first, K last: loads return in order, so once the K registers of a step have arrived (the
   // compiler waits for them before the first MFMA) the V strip of that step has landed too
   auto load_step = [&](vec8 (&kfr)[DS], int kv0, int stage) {
@@ -132,10 +134,10 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : NB == 1 ? (D == 64 ? 3 : 2) : (
     if constexpr (PASS != kDecLse) {
 #pragma unroll
       for (int j = 0; j < NVI; j++) {
-        const int r = RPI * j + fill_row;
-        const T* vg = vp + min(r, lim) * (int)vs2 + ((fill_pos ^ lds_swz<D>(r)) * 8);
+        const int c = 64 * j + lane, r = c / CPR;   // the strip row and position this lane fills
+        const T* vg = vp + min(r, lim) * (int)vs2 + (((c % CPR) ^ lds_swz<D>(r)) * 8);
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                         (__attribute__((address_space(3))) void*)(Vw + stage * kStripElems + RPI * j * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Vw + stage * kStripElems + 512 * j), 16, 0, 0);
       }
     }
     const T* kp = kbase + (int64_t)kv0 * ks2 + min(i32, lim) * (int)ks2 + 8 * g;
@@ -440,10 +442,10 @@ template <typename T, int D, int KIND, bool RS, int PASS>
 static void launch_nb(const FlexAttnParams& p, const DecodeArgs& a) {
   dim3 grid(a.splits, p.Hkv, p.B);
   const int ncols = (p.Hq / p.Hkv) * p.Lq;
-  if (ncols <= 32 || D == 256) {  // the caller has checked that D = 256 comes with at most 32 columns
+  if (ncols <= 32 || D >= 192) {  // the caller has checked that D = 192 / 256 come with at most 32 columns
     hipLaunchKernelGGL((decode_split_kernel<T, D, KIND, RS, 1, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
                        (const T*)a.v, a.o_part, a.ml_part, a.splits, a.lse_pass);
-  } else if constexpr (D != 256) {
+  } else if constexpr (D < 192) {
     hipLaunchKernelGGL((decode_split_kernel<T, D, KIND, RS, 2, PASS>), grid, dim3(256), 0, a.s, p, (const T*)a.q, (const T*)a.k,
                        (const T*)a.v, a.o_part, a.ml_part, a.splits, a.lse_pass);
   }

@@ -1,4 +1,4 @@
-// Split-KV decode for gfx950: short queries (G * Lq <= 64 columns; 32 at D = 256) against a
+// Split-KV decode for gfx950: short queries (G * Lq <= 64 columns; 32 at D = 192 / 256) against a
 // long KV cache, bound by HBM bandwidth.
 //
 // Serves the decode shapes of examples/benchmark_decoding.py:29-33 (the
@@ -31,16 +31,19 @@ int flex_decode_f16_64(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_f16_128(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_64(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_128(const FlexAttnParams& p, const DecodeArgs& a);
+int flex_decode_f16_192(const FlexAttnParams& p, const DecodeArgs& a);
+int flex_decode_bf16_192(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_f16_256(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_256(const FlexAttnParams& p, const DecodeArgs& a);
 void flex_set_error(const char* fmt, ...);
 bool flex_mfma_shape_ok(const FlexAttnParams& p);
 
-// 16-bit inputs, D = Dv in {64, 128} with up to 64 query columns (rows x heads per KV head) or D = Dv = 256 with up to 32
+// 16-bit inputs, D = Dv in {64, 128} with up to 64 query columns (rows x heads per KV head) or D = Dv in {192, 256}
+// with up to 32
 bool flex_decode_supported(const FlexAttnParams& p) {
   if (p.score.kind == FLEX_SCORE_AFFINE) return false;
   int max_cols = 64;
-  if (p.D == 256 && p.Dv == 256) {
+  if (p.D == p.Dv && (p.D == 192 || p.D == 256)) {
     FlexAttnParams as128 = p;  // dtype, stride and grid checks are those of the narrower heads
     as128.D = as128.Dv = 128;
     if (!flex_mfma_shape_ok(as128)) return false;
@@ -112,8 +115,10 @@ int flex_decode_launch(const FlexAttnParams& p, const void* q, const void* k, co
   float* lse_ws = ml_part + rows * splits * 2;
   const DecodeArgs a = {q, k, v, o, lse2, lse2 ? lse2 : lse_ws, o_part, ml_part, splits, s};
   int rc;
-  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_decode_f16_64(p, a) : p.D == 128 ? flex_decode_f16_128(p, a) : flex_decode_f16_256(p, a);
-  else rc = p.D == 64 ? flex_decode_bf16_64(p, a) : p.D == 128 ? flex_decode_bf16_128(p, a) : flex_decode_bf16_256(p, a);
+  if (p.dtype == FLEX_F16)
+    rc = p.D == 64 ? flex_decode_f16_64(p, a) : p.D == 128 ? flex_decode_f16_128(p, a) : p.D == 192 ? flex_decode_f16_192(p, a) : flex_decode_f16_256(p, a);
+  else
+    rc = p.D == 64 ? flex_decode_bf16_64(p, a) : p.D == 128 ? flex_decode_bf16_128(p, a) : p.D == 192 ? flex_decode_bf16_192(p, a) : flex_decode_bf16_256(p, a);
   if (rc) flex_set_error("decode: unsupported score_mod kind %d", p.score.kind);
   return rc;
 }

@@ -23,7 +23,7 @@ size_t flex_mfma_fwd_partial_bytes(const FlexAttnParams& p, int splits);
 int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, void* o, float* lse2, int splits,
                   void* partials, hipStream_t s);
 bool flex_mfma_bwd_supported(const FlexAttnParams& p);
-bool flex_mfma_dq256_supported(const FlexAttnParams& p);
+bool flex_mfma_dq_wide_supported(const FlexAttnParams& p);
 size_t flex_mfma_bwd_workspace(const FlexAttnParams& p);
 int flex_mfma_bwd(const FlexAttnParams& p, const void* q, const void* k, const void* v, const void* o, const float* lse2,
                   const void* d_o, void* dq, void* dk, void* dv, void* workspace, hipStream_t s);
@@ -190,8 +190,8 @@ extern "C" int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* 
   int rc;
   if (wants_fused(p) && flex_simple_supported(*p, 1)) {
     FlexAttnParams ps = with_parity_resolved(p, true);
-    if (flex_mfma_dq256_supported(ps) && !(ps.flags & (FLEX_BWD_ONLY_DQ | FLEX_BWD_ONLY_DKV))) {
-      // 256-wide heads: dQ (and the row sweep for delta, which the dK/dV kernel reads from the workspace) on the tuned
+    if (flex_mfma_dq_wide_supported(ps) && !(ps.flags & (FLEX_BWD_ONLY_DQ | FLEX_BWD_ONLY_DKV))) {
+      // 192- and 256-wide heads: dQ (and the row sweep for delta, which the dK/dV kernel reads from the workspace) on the tuned
       // kernel, dK/dV on the simple one
       FlexAttnParams pq = ps;
       pq.flags |= FLEX_BWD_ONLY_DQ;
@@ -228,7 +228,7 @@ extern "C" int flexattn_decode_static(const FlexAttnParams* p, const void* q, co
                                       float* lse2, int32_t num_splits, flexattn_stream_t stream) {
   if (int rc = validate(p, "flexattn_decode_static")) return rc;
   if (!flex_decode_supported(*p)) {
-    flex_set_error("flexattn_decode_static: needs fp16/bf16 and D == Dv in {64,128} with at most 64 query columns or D == Dv == 256 with at most 32 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
+    flex_set_error("flexattn_decode_static: needs fp16/bf16 and D == Dv in {64,128} with at most 64 query columns or D == Dv in {192,256} with at most 32 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
     return 1;
   }
   if (num_splits <= 0) num_splits = flex_decode_default_splits(*p);
@@ -251,7 +251,7 @@ static int decode_checked(const FlexAttnParams* p, const void* q, const void* k,
   if (p->q_index_base < 0) { flex_set_error("flexattn_decode: q_index_base must not be negative (got %d)", p->q_index_base); return 1; }
   if (!q || !k || !v || !o || !workspace) { flex_set_error("flexattn_decode: null pointer"); return 1; }
   if (!flex_decode_supported(*p)) {
-    flex_set_error("flexattn_decode: needs fp16/bf16 and D == Dv in {64,128} with at most 64 query columns or D == Dv == 256 with at most 32 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
+    flex_set_error("flexattn_decode: needs fp16/bf16 and D == Dv in {64,128} with at most 64 query columns or D == Dv in {192,256} with at most 32 (got dtype=%d D=%d Dv=%d Lq=%d)", p->dtype, p->D, p->Dv, p->Lq);
     return 1;
   }
   if (num_splits <= 0) num_splits = flex_decode_default_splits(*p);

@@ -45,7 +45,7 @@ enum { kFwdOnePass = 0, kFwdLse = 1, kFwdNorm = 2, kFwdHiLo = 3 };
 // D = 256: one wave per SIMD (Q fragments, K fragments and the accumulator are 64 + 64 + 128 registers, the V
 // fragments another 64 that are fetched late) and the two stages are 128 KB.
 template <typename T, int D, int KIND, bool ROUND_S, bool BITS, int PASS = kFwdOnePass>
-__global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
+__global__ __launch_bounds__(256, D >= 192 ? 1 : 2) void fwd_mfma_kernel(FlexAttnParams p, const T* __restrict__ q,
                                                            const T* __restrict__ k, const T* __restrict__ v,
                                                            T* __restrict__ o, float* __restrict__ lse2,
                                                            float* __restrict__ o_part, float* __restrict__ ml_part) {
@@ -59,9 +59,10 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
   constexpr int DS = D / 16;     // k-steps of the Q.K^T product
   constexpr int DB = D / 32;     // 32-row blocks of O^T
   constexpr int CPR = D / 8;     // 16-byte chunks per row
-  constexpr int RPI = 64 / CPR;        // rows one wave-wide fetch instruction fills
-  constexpr int NI = (BN / 4) / RPI;   // fetch instructions per wave, tile and tensor (a wave fills 16 rows = one swizzle period)
-  static_assert((BN / 4) == 16, "a wave's share of a tile is one swizzle period");
+  // a wave fills 16 rows (one swizzle period) of a tile: 16 * CPR chunks, 64 per fetch instruction, laid down one after
+  // the other; at D = 192 an instruction ends in the middle of a row
+  constexpr int NI = 16 * CPR / 64;    // fetch instructions per wave, tile and tensor
+  static_assert((BN / 4) == 16 && (16 * CPR) % 64 == 0, "a wave's share of a tile is one swizzle period");
   // two LDS stages, filled straight from global memory (no staging registers, unpadded swizzled rows): while one
   // tile is consumed the next one lands, one workgroup barrier per tile.  Each stage is a variable of its own and
   // every access names its stage at compile time (the tile loop is unrolled by two): only then can the compiler
@@ -130,13 +131,11 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
   // fills position (r, pos) fetches chunk pos ^ lds_swz(r) of that row.  The per-lane part of a fetch address (row
   // inside the swizzle period, swizzled chunk) is the same for every tile: kept as byte offsets from a wave-uniform
   // row address.
-  const int fill_row = lane / CPR, fill_pos = lane % CPR;
   const int wu = __builtin_amdgcn_readfirstlane(w);
   uint32_t koff[NI], voff[NI];
 #pragma unroll
   for (int j = 0; j < NI; j++) {
-    const int row = RPI * j + fill_row;
-    const int chunk = fill_pos ^ lds_swz<D>(row);
+    const int c = 64 * j + lane, row = c / CPR, chunk = (c % CPR) ^ lds_swz<D>(row);
     koff[j] = (uint32_t)((row * ks2 + chunk * 8) * (int64_t)sizeof(T));
     voff[j] = (uint32_t)((row * vs2 + chunk * 8) * (int64_t)sizeof(T));
   }
@@ -152,24 +151,24 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
 #pragma unroll
       for (int j = 0; j < NI; j++) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(kt + koff[j]),
-                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * j) * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D + 512 * j), 16, 0, 0);
         if constexpr (PASS != kFwdLse)
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(vt + voff[j]),
-                                           (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * j) * D), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void*)(Vst + r0 * D + 512 * j), 16, 0, 0);
       }
     } else {
       // the last tile of a ragged length: rows past the end are clamped (finite filler, masked out below)
 #pragma unroll
       for (int j = 0; j < NI; j++) {
-        const int chunk = fill_pos ^ lds_swz<D>(RPI * j + fill_row);
-        const int row = min(r0 + RPI * j + fill_row, lim);
+        const int c = 64 * j + lane, rw = c / CPR, chunk = (c % CPR) ^ lds_swz<D>(rw);
+        const int row = min(r0 + rw, lim);
         const T* kg = kbase + (int64_t)(kv0 + row) * ks2 + chunk * 8;
         const T* vg = vbase + (int64_t)(kv0 + row) * vs2 + chunk * 8;
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)kg,
-                                         (__attribute__((address_space(3))) void*)(Kst + (r0 + RPI * j) * D), 16, 0, 0);
+                                         (__attribute__((address_space(3))) void*)(Kst + r0 * D + 512 * j), 16, 0, 0);
         if constexpr (PASS != kFwdLse)
           __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)vg,
-                                           (__attribute__((address_space(3))) void*)(Vst + (r0 + RPI * j) * D), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void*)(Vst + r0 * D + 512 * j), 16, 0, 0);
       }
     }
   };
@@ -257,7 +256,7 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
         for (int s = 0; s < DS; s++) kfr[s] = *reinterpret_cast<const vec8*>(kp + (((2 * s) ^ kz) * 8));
         // (D = 256: the 64 registers of V fragments are fetched right before their product instead, or the block
         // would not fit a wave's registers)
-        if constexpr (PASS != kFwdLse && D != 256) {
+        if constexpr (PASS != kFwdLse && D < 192) {
 #pragma unroll
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
@@ -374,7 +373,7 @@ __global__ __launch_bounds__(256, D == 256 ? 1 : 2) void fwd_mfma_kernel(FlexAtt
           for (int tt = 0; tt < 2; tt++)
 #pragma unroll
             for (int db = 0; db < DB; db++) {
-              if constexpr (D == 256) {
+              if constexpr (D >= 192) {
                 const T* vp = Vs + (32 * nb + 16 * tt) * D;
                 vfr[tt][db] = join8<vec8>(lds_read_tr(vp + toff[0][db]), lds_read_tr(vp + toff[1][db]));
               }

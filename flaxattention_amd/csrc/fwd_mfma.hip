@@ -1,4 +1,4 @@
-// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128, 256}): checks and dispatch.  The kernels
+// Fused flash-attention forward for gfx950 (fp16 / bf16, D = Dv in {64, 128, 192, 256}): checks and dispatch.  The kernels
 // are in fwd_mfma.cuh, instantiated per (dtype, head size) by fwd_mfma_inst.hip.
 #include "fwd_mfma.cuh"
 
@@ -8,6 +8,8 @@ int flex_mfma_fwd_f16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_f16_128(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_128(const FlexAttnParams& p, const FwdArgs& a);
+int flex_mfma_fwd_f16_192(const FlexAttnParams& p, const FwdArgs& a);
+int flex_mfma_fwd_bf16_192(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_f16_256(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_256(const FlexAttnParams& p, const FwdArgs& a);
 
@@ -35,9 +37,9 @@ void flex_mfma_tiles(int dtype, int D, int Dv, int which, int* qb, int* kvb) {
 }
 
 bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
-  if (p.D == 256 && p.Dv == 256) {
-    // the list-driven forward is also instantiated for 256-wide heads (one wave per SIMD); everything but the head
-    // size is checked as for 128
+  if (p.D == p.Dv && (p.D == 192 || p.D == 256)) {
+    // the list-driven forward is also instantiated for 192- and 256-wide heads (one wave per SIMD); everything but
+    // the head size is checked as for 128
     FlexAttnParams as128 = p;
     as128.D = as128.Dv = 128;
     if (!flex_mfma_shape_ok(as128)) return false;
@@ -54,7 +56,7 @@ bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
 // keys each.
 int flex_mfma_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B;
-  const int slots = p.D == 256 ? 256 : 512;  // 256-wide heads run one workgroup per compute unit
+  const int slots = p.D >= 192 ? 256 : 512;  // 192- and 256-wide heads run one workgroup per compute unit
   if (wgs > slots / 2) return 1;
   const int tiles = (p.Lkv + kFwdBN - 1) / kFwdBN;
   int s = (int)(slots / wgs);
@@ -90,8 +92,10 @@ int flex_mfma_fwd(const FlexAttnParams& p, const void* q, const void* k, const v
     a.ml_part = a.o_part + (size_t)p.B * p.Hq * p.Lq * splits * p.D;
   }
   int rc = 1;
-  if (p.dtype == FLEX_F16) rc = p.D == 64 ? flex_mfma_fwd_f16_64(p, a) : p.D == 128 ? flex_mfma_fwd_f16_128(p, a) : flex_mfma_fwd_f16_256(p, a);
-  else rc = p.D == 64 ? flex_mfma_fwd_bf16_64(p, a) : p.D == 128 ? flex_mfma_fwd_bf16_128(p, a) : flex_mfma_fwd_bf16_256(p, a);
+  if (p.dtype == FLEX_F16)
+    rc = p.D == 64 ? flex_mfma_fwd_f16_64(p, a) : p.D == 128 ? flex_mfma_fwd_f16_128(p, a) : p.D == 192 ? flex_mfma_fwd_f16_192(p, a) : flex_mfma_fwd_f16_256(p, a);
+  else
+    rc = p.D == 64 ? flex_mfma_fwd_bf16_64(p, a) : p.D == 128 ? flex_mfma_fwd_bf16_128(p, a) : p.D == 192 ? flex_mfma_fwd_bf16_192(p, a) : flex_mfma_fwd_bf16_256(p, a);
   if (rc) flex_set_error("fused forward: unsupported score_mod kind %d", p.score.kind);
   return rc;
 }

@@ -523,8 +523,11 @@ __device__ __forceinline__ int uniform_ld(const int32_t* ptr) {
 //     must land in different 64-byte quarters of the period.
 // D = 64 (128-byte rows, two per period): bit 2 of the chunk follows bit 1 of r, bits 0-1 follow
 // bits 2-3.  D = 128 (one row per period): bits 2-3 follow bits 0-1 of r, bits 0-1 follow bits 2-3.
+// D = 192 (384-byte rows, one and a half periods: odd rows start half a period in, which supplies bit 3 of the
+// slot): only the low three bits may move, or a chunk would leave its row of 24; bit 2 follows bit 1 of r, bits 0-1
+// follow bits 2-3.  D = 256 (two periods per row) takes the D = 128 rule.
 template <int D> __device__ __forceinline__ constexpr int lds_swz(int r) {
-  return D == 64 ? (((r & 2) << 1) | ((r >> 2) & 3)) : (((r & 3) << 2) | ((r >> 2) & 3));
+  return (D == 64 || D == 192) ? (((r & 2) << 1) | ((r >> 2) & 3)) : (((r & 3) << 2) | ((r >> 2) & 3));
 }
 
 // XCD-aware, heavy-first workgroup map.  Hardware deals consecutive workgroup ids

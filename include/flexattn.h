@@ -229,7 +229,7 @@ int flexattn_bwd(const FlexAttnParams* p, const void* q, const void* k, const vo
                  void* dq, void* dk, void* dv, void* workspace, flexattn_stream_t stream);
 
 /* Split-KV decode for short queries: fp16 / bf16, D = Dv in {64, 128} with at most 64 query
- * columns (query rows x query heads per KV head) or D = Dv = 256 with at most 32.  Replaces the
+ * columns (query rows x query heads per KV head) or D = Dv in {192, 256} with at most 32.  Replaces the
  * same reference functions as flexattn_fwd for the decode shapes of
  * examples/benchmark_decoding.py:29-33.  num_splits <= 0 picks a default.  */
 size_t flexattn_decode_workspace_bytes(const FlexAttnParams* p, int32_t num_splits);

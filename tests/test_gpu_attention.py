@@ -565,13 +565,14 @@ def test_fused_unrounded_numerics(dev, dtype, D, name, score, oscore):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
-def test_unrounded_numerics_at_256(dev, dtype):
-    """256-wide heads in the "unrounded" numerics: the forward runs on the list-driven matrix-core kernel (P in high and
-    low parts), the backward on the vector-ALU kernels; both against the oracle without round trips."""
+@pytest.mark.parametrize("D", [192, 256])
+def test_unrounded_numerics_at_wide_heads(dev, dtype, D):
+    """192- and 256-wide heads in the "unrounded" numerics: the forward runs on the list-driven matrix-core kernel (P in
+    high and low parts), the backward on the vector-ALU kernels; both against the oracle without round trips."""
     name, score, oscore = SCORES[4]
     assert name == "alibi_cfg"
-    test_fused_unrounded_numerics(dev, dtype, 256, name, score, oscore)
-    q, k, v = (t.to(dev) for t in seeded_qkv(2, 4, 2, 256, 320, 256, dtype))
+    test_fused_unrounded_numerics(dev, dtype, D, name, score, oscore)
+    q, k, v = (t.to(dev) for t in seeded_qkv(2, 4, 2, 256, 320, D, dtype))
     assert fa.kernel_family(q, k, v, kernel_options={"numerics": "unrounded"}) == "mfma_16bit"
     assert fa.kernel_family(q, k, v, kernel_options={"numerics": "unrounded"}, backward=True) == "generic"
 

@@ -59,19 +59,22 @@ def test_decode_parity_numerics(dev, dtype, Lq, D, splits):
 @pytest.mark.parametrize("dtype,numerics", [(torch.float16, None), (torch.bfloat16, None), (torch.bfloat16, "fast"),
                                             (torch.float16, "parity")], ids=["f16", "bf16", "bf16-fast", "f16-parity"])
 @pytest.mark.parametrize("Lq,G,splits", [(1, 1, 8), (7, 4, 3), (32, 1, 5), (2, 16, 1)])
-def test_decode_256_wide_heads(dev, dtype, numerics, Lq, G, splits):
-    """D = 256: one column block (at most 32 columns); ALiBi + offset-causal with a ragged KV length, GQA packing."""
+@pytest.mark.parametrize("D", [192, 256])
+def test_decode_wide_heads(dev, dtype, numerics, Lq, G, splits, D):
+    """D = 192 / 256: one column block (at most 32 columns); ALiBi + offset-causal with a ragged KV length, GQA packing."""
     Lkv, Hkv = 1237, 2
-    run_decode(dev, dtype, 2, Hkv * G, Hkv, Lq, Lkv, 256, splits, generate_alibi_bias(Hkv * G, -1.0), o_alibi_config(Hkv * G),
+    run_decode(dev, dtype, 2, Hkv * G, Hkv, Lq, Lkv, D, splits, generate_alibi_bias(Hkv * G, -1.0), o_alibi_config(Hkv * G),
                offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq), numerics=numerics)
 
 
-def test_decode_256_wide_heads_choice_and_chunks(dev):
-    """D = 256 is routed to the decode kernel up to 32 columns per call; longer queries go there in chunks of 32 rows
-    on request; the library refuses more than 32 columns in one call and the results agree with the forward kernel."""
+@pytest.mark.parametrize("D", [192, 256])
+def test_decode_wide_heads_choice_and_chunks(dev, D):
+    """D = 192 / 256 are routed to the decode kernel up to 32 columns per call; longer queries go there in chunks of 32
+    rows on request; the library refuses more than 32 columns in one call and the results agree with the forward
+    kernel."""
     from flaxattention_amd.core.attention import _make_plan
     from flaxattention_amd import _lib
-    B, H, Lq, Lkv, D = 1, 2, 80, 4096, 256
+    B, H, Lq, Lkv = 1, 2, 80, 4096
     q, k, v = seeded_qkv(B, H, H, Lq, Lkv, D, torch.float16)
     mask, omask = offset_causal_mask(Lkv - Lq), o_offset_causal(Lkv - Lq)
     bm = fa.create_block_mask(mask, B, H, Lq, Lkv, device=dev)
@@ -83,7 +86,7 @@ def test_decode_256_wide_heads_choice_and_chunks(dev):
                                  kernel_options={"decode": True})
     want, want_lse = ref_attention(q, k, v, o_alibi_config(H), omask, strict=True, return_lse=True)
     a, r = max_abs(out.cpu(), want), rel_l2(out.cpu(), want)
-    print(f"  chunked decode at D=256 O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
+    print(f"  chunked decode at D={D} O: max-abs {a:.3e} rel-L2 {r:.3e}", flush=True)
     assert a <= 2e-2 and r <= 1e-3
     assert max_abs(lse.cpu(), want_lse) <= 2e-2
     ref = fa.flax_attention(qd, kd, vd, score_mod=generate_alibi_bias(H, -1.0), block_mask=bm, kernel_options={"decode": False})

@@ -104,8 +104,8 @@ def test_forward_backward_against_faithful_kernels(dev, seed):
 def test_decode_chunks_and_split_forward_against_faithful_kernels(dev, seed):
     r = random.Random(1000 + seed)
     dtype = r.choice([torch.float16, torch.bfloat16])
-    D = r.choice([64, 128, 256])
-    cols = 32 if D == 256 else 64
+    D = r.choice([64, 128, 192, 256])
+    cols = 32 if D >= 192 else 64
     B, Hkv, G = r.randint(1, 3), r.randint(1, 3), r.choice([1, 1, 2, 4, 8])
     Hq = Hkv * G
     mode = r.choice(["decode", "decode", "chunks", "split_forward"])
