@@ -11,8 +11,8 @@ printed on stdout is ONE JSON object (the driver's contract).  Besides the
 headline it carries the decode half of the metric (configuration 5, q_len 1,
 16 and 64 over rotating KV caches: us, GB/s, fraction of 8 TB/s), the step
 times of configurations 3 and 4, and every training configuration in the three
-numerics modes ("fast", "parity", "unrounded"); --all adds the probes, the split sweep
-of the decode kernel and the block-mask builder.
+numerics modes ("fast", "parity", "unrounded"); --all adds the split sweep of the decode
+kernel and the block-mask builder.
 
 Kernel durations are HIP-event intervals taken INSIDE the step (forward, dQ
 and dK/dV launched in their real order, an event between them): a kernel
@@ -222,10 +222,37 @@ def make_train_config(dev, name, opts=None):
         # the configuration's spelling of the checkerboard: x0.5 where kv_idx is odd, x2.0 where even; no mask
         pr = Prepared(dev, torch.float16, 8, 8, 8, 2048, 2048, 64, generate_checkerboard(2.0, 0.5, "kv"), None, opts)
         tiles, dtype = 8 * 8 * tiles_128("none", 2048), "fp16"
+    elif name == "config2_causal":
+        # the combination the target sentence names: configuration 2's checkerboard under a causal block mask
+        pr = Prepared(dev, torch.float16, 8, 8, 8, 2048, 2048, 64, generate_checkerboard(2.0, 0.5, "kv"), causal_mask, opts)
+        tiles, dtype = 8 * 8 * tiles_128("causal", 2048), "fp16"
     else:
         pr = Prepared(dev, torch.bfloat16, 8, 8, 8, 2048, 2048, 64, generate_alibi_bias(8, -1.0), causal_mask, opts)
         tiles, dtype = 8 * 8 * tiles_128("causal", 2048), "bf16"
     return pr, tiles, dtype
+
+
+def run_api_step(dev, steps, warmup):
+    """Configuration 2 as a caller of the drop-in sees it: flax_attention(...) and .backward() on torch tensors,
+    with everything the front end does per call (lowering lookups, parameter block, output and workspace allocation,
+    autograd) inside the timed region.  Two spellings of the same gradient: backward(ones), and out.sum().backward()
+    as the reference's benchmark script writes it (which adds torch's reduction and the materialised cotangent)."""
+    import flaxattention_amd as fa
+    from flaxattention_amd.mods import generate_checkerboard
+    g = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda *s: torch.randn(*s, generator=g, dtype=torch.float32, device=dev).to(torch.float16).requires_grad_(True)
+    k, q, v = mk(8, 8, 2048, 64), mk(8, 8, 2048, 64), mk(8, 8, 2048, 64)
+    d_o = torch.ones(8, 8, 2048, 64, dtype=torch.float16, device=dev)
+    score = generate_checkerboard(2.0, 0.5, "kv")
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        fa.flax_attention(q, k, v, score_mod=score).backward(d_o)
+
+    def step_sum():
+        q.grad = k.grad = v.grad = None
+        fa.flax_attention(q, k, v, score_mod=score).sum().backward()
+    return {"api_ms_per_step": wall_time_ms(step, steps, warmup), "api_sum_backward_ms_per_step": wall_time_ms(step_sum, steps, warmup)}
 
 
 def run_train_config(dev, name, steps, warmup, opts=None, graph=False):
@@ -292,97 +319,6 @@ def pmc_probe(dev, name, opts):
         for _ in range(3):
             pd.decode()
     torch.cuda.synchronize()
-
-
-_probe_lib = None
-
-
-def probe_lib():
-    """libflexprobe.so: bench-only measurement kernels (MFMA-only, instruction-mix and streaming-read), built next to
-    the product library by the same Makefile but no part of it."""
-    global _probe_lib
-    if _probe_lib is None:
-        from flaxattention_amd import _lib
-        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "libflexprobe.so")
-        L = C.CDLL(path)
-        L.flexprobe_last_error.restype = C.c_char_p
-        L.flexprobe_mfma.argtypes = [C.c_void_p, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
-        L.flexprobe_mix.argtypes = [C.c_void_p, C.c_int32, C.c_int32, C.POINTER(C.c_double), C.c_void_p]
-        L.flexprobe_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]
-        _probe_lib = L
-    return _probe_lib
-
-
-def probe_check(rc, who):
-    if rc:
-        raise RuntimeError(f"{who} failed ({rc}): {probe_lib().flexprobe_last_error().decode()}")
-
-
-def run_mfma_probe(dev):
-    """Matrix throughput this GPU sustains on a kernel that only issues fp16 MFMAs on pseudo-random operands:
-    the practical ceiling next to the published peak."""
-    L = probe_lib()
-    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
-    flops = C.c_double(0.0)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-
-    def go():
-        probe_check(L.flexprobe_mfma(sink.data_ptr(), 4096, C.byref(flops), stream), "flexprobe_mfma")
-    us = event_time_us(go, 20)
-    return flops.value / us / 1e6
-
-
-def run_mix_probe(dev):
-    """Matrix flop rate of the instruction-mix probe: 8, 12 or 16 MFMAs interleaved with the vector work of
-    one 32x32 score block (80 FMAs + 16 exponentials), two waves per SIMD.  The ceiling of a fused attention step of
-    that mix on this GPU: 8 = forward at D 64, 12 = dQ kernel, 16 = dK/dV kernel and forward at D 128."""
-    L = probe_lib()
-    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
-    flops = C.c_double(0.0)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    out = {}
-    for nm in (8, 12, 16):
-        def go():
-            probe_check(L.flexprobe_mix(sink.data_ptr(), 2048, nm, C.byref(flops), stream), "flexprobe_mix")
-        us = event_time_us(go, 20)
-        out[str(nm)] = round(flops.value / us / 1e6, 1)
-    return out
-
-
-def run_read_probe(dev):
-    """Read rate of the bare streaming-read kernel, GB/s.  (a) 268 MB (the K + V bytes of one decode call of
-    configuration 5) rotating over three buffers, which no launch finds in the 256 MB last-level cache, and
-    re-reading one buffer; (b) the same kernel over 2 GiB at several grid sizes and loads in flight per thread: at
-    that size launch ramp and tail are under 2 % of the run, so the best of these is the steady-state read rate of
-    the memory system, against which the 268 MB figure shows what a 50 us kernel loses to ramp and tail."""
-    L = probe_lib()
-    nbytes = 2 * 8 * 8 * 16384 * 64 * 2
-    bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(3)]
-    sink = torch.zeros(65536, dtype=torch.float32, device=dev)
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    turn = [0]
-
-    def go(n_bufs, wgs=0, nld=0):
-        rc = L.flexprobe_read(bufs[turn[0] % n_bufs].data_ptr(), nbytes, sink.data_ptr(), wgs, nld, stream)
-        turn[0] += 1
-        probe_check(rc, "flexprobe_read")
-    out = {"rotating_buffers": round(nbytes / event_time_us(lambda: go(3), 30) / 1e3),
-           "one_buffer": round(nbytes / event_time_us(lambda: go(1), 30) / 1e3)}
-    shapes = {}
-    for wgs in (512, 1024, 2048, 4096, 8192):
-        for nld in (2, 4, 8, 16):
-            shapes[f"{wgs}x{nld}"] = round(nbytes / event_time_us(lambda: go(3, wgs, nld), 15) / 1e3)
-    out["rotating_268MB_by_workgroups_x_loads"] = shapes
-    del bufs
-    big = torch.randint(0, 255, (2 << 30,), dtype=torch.uint8, device=dev)
-    steady = {}
-    for wgs in (1024, 2048, 4096, 8192):
-        for nld in (4, 8, 16):
-            def one():
-                probe_check(L.flexprobe_read(big.data_ptr(), big.numel(), sink.data_ptr(), wgs, nld, stream), "flexprobe_read")
-            steady[f"{wgs}x{nld}"] = round(big.numel() / event_time_us(one, 5, warm=1) / 1e3)
-    out["steady_2GiB_by_workgroups_x_loads"] = steady
-    return out
 
 
 def run_block_mask_build(dev):
@@ -456,7 +392,7 @@ def main():
     ap.add_argument("--workload", default="config2", choices=["config2", "config3"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--headline-only", action="store_true", help="only the headline workload (no other configurations, modes or decode)")
-    ap.add_argument("--all", action="store_true", help="also the probes, the decode split sweep and the block-mask builder (in 'extra')")
+    ap.add_argument("--all", action="store_true", help="also the decode split sweep and the block-mask builder (in 'extra')")
     ap.add_argument("--round-s", type=int, default=1, help="round Q.K^T through the input dtype (default 1)")
     ap.add_argument("--numerics", default=None, choices=["fast", "parity", "unrounded"],
                     help="numerics of the headline workload (default: the library's: fp16 fast, bf16 parity)")
@@ -513,6 +449,13 @@ def main():
                 log(f"{wl} numerics {num}: {rr['ms_per_step'] * 1e3:.1f} us/step  {rr['tflops']:.1f} TFLOP/s  {modes[wl][num]['kernels_us']}")
         modes["config4"] = c4
         line_extra["numerics_modes"] = modes
+        rc = run_train_config(dev, "config2_causal", a.steps, a.warmup, opts)
+        line_extra["config2_causal"] = dict(mode_summary(rc), workload="fp16 [8,8,2048,64] checkerboard score_mod under a causal block mask "
+                                            "(128x128), forward + backward of out.sum(); flops of the 136 of 256 visible tiles per head")
+        log(f"config2 + causal: {rc['ms_per_step'] * 1e3:.1f} us/step  {rc['tflops']:.1f} TFLOP/s  {line_extra['config2_causal']['kernels_us']}")
+        api = run_api_step(dev, a.steps, a.warmup)
+        line_extra["api"] = {k: round(v, 5) for k, v in api.items()}
+        log(f"configuration 2 through flax_attention + backward: {api}")
     # The headline comes last: by now the GPU has been under load for seconds.  Started from idle, the first ~50
     # steps (20 ms) run through a transient of the power management (step times of 370 -> 530 -> 360 us in a kernel
     # trace); W warm-up steps and K timed steps placed there would measure that transient, not the sustained rate.
@@ -521,15 +464,6 @@ def main():
         f"(fwd {r['fwd_tflops']:.1f}, bwd {r['bwd_tflops']:.1f})  kernels {r['kernels']}")
     extra = {}
     if a.all:
-        probe = run_mfma_probe(dev)
-        log(f"MFMA-only probe kernel (fp16, pseudo-random operands): {probe:.0f} TFLOP/s sustained")
-        extra["mfma_probe_tflops"] = round(probe, 1)
-        mix = run_mix_probe(dev)
-        log(f"instruction-mix probe (MFMAs per 96 vector instructions -> matrix TFLOP/s): {mix}")
-        extra["mix_probe_tflops"] = mix
-        rd = run_read_probe(dev)
-        log(f"bare read: {rd}")
-        extra["read_probe_gbps"] = rd
         bmb = run_block_mask_build(dev)
         log(f"create_block_mask: {bmb} us")
         extra["block_mask_build_us"] = bmb

@@ -265,6 +265,23 @@ def affine_score_mod(fn: Callable, B: int, H: int, Lq: int, Lkv: int, device) ->
         add = add.unsqueeze(0)
     while mul.dim() < 4:
         mul = mul.unsqueeze(0)
+    if not (bool(torch.isfinite(add).all()) and bool(torch.isfinite(mul).all())):
+        return None
+    # The corner grid only says that the callable is affine near the origin of the index space.  The tables are
+    # accepted when they reproduce the callable at further scores on EVERY (b, h, q_idx, kv_idx) of the problem: a mod
+    # that is affine for the first keys, rows or batch entries and something else beyond them (a soft-cap past a few
+    # sink keys, a square for some batch index) must not be lowered to tables.  Row slabs bound the temporaries.
+    rows = max(1, min(Lq, _SLAB_ELEMS // max(1, B * H * Lkv)))
+    for q0 in range(0, Lq, rows):
+        qs = qi[:, :, q0:q0 + rows]
+        a_s = add[:, :, q0:q0 + rows] if add.shape[2] == Lq else add
+        m_s = mul[:, :, q0:q0 + rows] if mul.shape[2] == Lq else mul
+        for s_chk in (0.625, -1.75, 3.25):
+            got = torch.as_tensor(fn(zero + s_chk, bi, hi, qs, ki)).to(torch.float32)
+            while got.dim() < 4:
+                got = got.unsqueeze(0)
+            if not bool(torch.allclose(got, m_s * s_chk + a_s, rtol=1e-5, atol=1e-5)):
+                return None
     full = (B, H, Lq, Lkv)
     shp = tuple(max(add.shape[i], mul.shape[i]) for i in range(3)) + (Lkv,)
     if any(shp[i] not in (1, full[i]) for i in range(3)):

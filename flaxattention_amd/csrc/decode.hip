@@ -36,6 +36,7 @@ int flex_decode_bf16_192(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_f16_256(const FlexAttnParams& p, const DecodeArgs& a);
 int flex_decode_bf16_256(const FlexAttnParams& p, const DecodeArgs& a);
 void flex_set_error(const char* fmt, ...);
+int flex_cu_count();
 bool flex_mfma_shape_ok(const FlexAttnParams& p);
 
 // 16-bit inputs, D = Dv in {64, 128} with up to 64 query columns (rows x heads per KV head) or D = Dv in {192, 256}
@@ -60,7 +61,7 @@ int flex_decode_default_splits(const FlexAttnParams& p) {
   // 16; at q_len 64: 56 us with 4, 60 us with 8).  At least 8 steps each.
   const int steps = (p.Lkv + kStep - 1) / kStep;
   int64_t heads = (int64_t)p.B * p.Hkv;
-  const int slots = 256;
+  const int slots = flex_cu_count();
   int s = (int)((slots + heads - 1) / heads);
   if (s > steps / 8) s = steps / 8;
   if (s < 1) s = 1;

@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include "flex_common.cuh"
 
 static thread_local char g_err[512] = "";
@@ -11,6 +12,29 @@ void flex_set_error(const char* fmt, ...) {
   va_start(ap, fmt);
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
   va_end(ap);
+}
+
+// Compute units of the current device, asked once per device (the split heuristics size their grids by it).  Without
+// a usable device -- a size query on a machine that only builds -- the answer is the MI355X's 256.
+int flex_cu_count() {
+  constexpr int kMaxDev = 64, kDefault = 256;
+  static std::mutex mu;
+  static int cus_of[kMaxDev] = {};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) {
+    (void)hipGetLastError();
+    return kDefault;
+  }
+  std::lock_guard<std::mutex> lock(mu);
+  if (!cus_of[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      (void)hipGetLastError();
+      n = kDefault;
+    }
+    cus_of[dev] = n;
+  }
+  return cus_of[dev];
 }
 
 // implemented in the kernel translation units

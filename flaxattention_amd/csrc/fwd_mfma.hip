@@ -4,6 +4,7 @@
 
 using namespace flex;
 void flex_set_error(const char* fmt, ...);
+int flex_cu_count();
 int flex_mfma_fwd_f16_64(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_f16_128(const FlexAttnParams& p, const FwdArgs& a);
 int flex_mfma_fwd_bf16_64(const FlexAttnParams& p, const FwdArgs& a);
@@ -56,7 +57,7 @@ bool flex_mfma_fwd_supported(const FlexAttnParams& p) {
 // keys each.
 int flex_mfma_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kFwdBM - 1) / kFwdBM) * p.Hq * p.B;
-  const int slots = p.D >= 192 ? 256 : 512;  // 192- and 256-wide heads run one workgroup per compute unit
+  const int slots = (p.D >= 192 ? 1 : 2) * flex_cu_count();  // 192- and 256-wide heads run one workgroup per compute unit
   if (wgs > slots / 2) return 1;
   const int tiles = (p.Lkv + kFwdBN - 1) / kFwdBN;
   int s = (int)(slots / wgs);

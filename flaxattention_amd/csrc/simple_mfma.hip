@@ -4,6 +4,7 @@
 
 using namespace flex;
 void flex_set_error(const char* fmt, ...);
+int flex_cu_count();
 int flex_simple_f32_64(const FlexAttnParams& p, const SimpleArgs& a);
 int flex_simple_f32_128(const FlexAttnParams& p, const SimpleArgs& a);
 int flex_simple_f16_192(const FlexAttnParams& p, const SimpleArgs& a);
@@ -52,9 +53,10 @@ static int dispatch(const FlexAttnParams& p, const SimpleArgs& a) {
 // workgroup per compute unit, with at least 16 steps of 32 keys each.
 int flex_simple_fwd_splits(const FlexAttnParams& p) {
   const int64_t wgs = (int64_t)((p.Lq + kSimpleQTile - 1) / kSimpleQTile) * p.Hq * p.B;
-  if (wgs > 128) return 1;
+  const int cus = flex_cu_count();
+  if (wgs > cus / 2) return 1;
   const int steps = (p.Lkv + kSimpleStep - 1) / kSimpleStep;
-  int s = (int)(256 / wgs);
+  int s = (int)(cus / wgs);
   if (s > steps / 16) s = steps / 16;
   if (s > 64) s = 64;  // the merge kernel takes one split per lane
   return s < 2 ? 1 : s;

@@ -295,7 +295,13 @@ def _mods_for_slice(score_mod, mask_mod, b0, nb, Hq, M, N):
     return b, _idx(Hq, 1), _idx(M, 2), _idx(N, 3)
 
 
-def _forward_slice(q, k, v, score_mod, mask_mod, scale, strict, b0, want_grad_mod=False):
+# Test hook: deliberately WRONG placements of the 16-bit rounding points, so that the test that pins the
+# placement (tests/test_oracle_cpu.py::test_rounding_points_against_torch_half_program) can show that it
+# would notice each of them.  Never set outside that test.
+MUTANTS = ("s_after_scale", "p_unrounded", "dp_unrounded", "ds_unrounded")
+
+
+def _forward_slice(q, k, v, score_mod, mask_mod, scale, strict, b0, want_grad_mod=False, _mutant=None):
     """q,k,v: [nb,H,*,*] slices already GQA-expanded.  Returns fp32 tensors
     X (post-mod, -inf masked), P (normalised), lse (natural), and optionally
     dmod/dS."""
@@ -305,8 +311,11 @@ def _forward_slice(q, k, v, score_mod, mask_mod, scale, strict, b0, want_grad_mo
     N = k.shape[2]
     # attention.py:27 -- matmul in the input dtype, then cast to fp32
     S = torch.matmul(q.to(wp), k.to(wp).transpose(-1, -2))
-    S = _rt(S, dtype, strict)
-    S = S * scale                                    # attention.py:55
+    if _mutant == "s_after_scale":
+        S = _rt(S * scale, dtype, strict)
+    else:
+        S = _rt(S, dtype, strict)
+        S = S * scale                                # attention.py:55
     b, h, m, n = _mods_for_slice(score_mod, mask_mod, b0, nb, Hq, M, N)
     mask = mask_mod(b, h, m, n)                      # attention.py:57-58
     if not torch.is_tensor(mask):
@@ -337,7 +346,7 @@ def _expand_gqa(x, G):
 
 
 def ref_attention(q, k, v, score_mod=None, mask_mod=None, scale=None, strict=True,
-                  return_lse=False, batch_chunk: int = 1):
+                  return_lse=False, batch_chunk: int = 1, _mutant=None):
     """flax_attention (attention.py:169-218) on CPU.  ``mask_mod`` is the
     scalar mask function (the only field of the block mask the reference's
     dense path reads, attention.py:45).  Returns O in the input dtype and,
@@ -353,8 +362,8 @@ def ref_attention(q, k, v, score_mod=None, mask_mod=None, scale=None, strict=Tru
     for b0 in range(0, q.shape[0], batch_chunk):
         sl = slice(b0, b0 + batch_chunk)
         kk, vv = _expand_gqa(k[sl], G), _expand_gqa(v[sl], G)
-        _, P, lse, _, _ = _forward_slice(q[sl], kk, vv, score_mod, mask_mod, scale, strict, b0)
-        O = torch.matmul(_rt(P, dtype, strict), vv.to(wp))          # attention.py:105
+        _, P, lse, _, _ = _forward_slice(q[sl], kk, vv, score_mod, mask_mod, scale, strict, b0, _mutant=_mutant)
+        O = torch.matmul(_rt(P, dtype, strict and _mutant != "p_unrounded"), vv.to(wp))          # attention.py:105
         outs.append(O.to(dtype))
         lses.append(lse)
     O = torch.cat(outs, 0)
@@ -364,7 +373,7 @@ def ref_attention(q, k, v, score_mod=None, mask_mod=None, scale=None, strict=Tru
 
 
 def ref_attention_bwd(q, k, v, dO, score_mod=None, mask_mod=None, scale=None, strict=True,
-                      batch_chunk: int = 1):
+                      batch_chunk: int = 1, _mutant=None):
     """Gradients (dQ, dK, dV) of sum(O * dO) for ref_attention, i.e. what
     jax.grad yields through attention.py:14-106 with the dtype round trips of
     the forward transposed: dP and dS pass through the input dtype in strict
@@ -383,14 +392,14 @@ def ref_attention_bwd(q, k, v, dO, score_mod=None, mask_mod=None, scale=None, st
         kk, vv = _expand_gqa(k[sl], G), _expand_gqa(v[sl], G)
         qq, dd = q[sl], dO[sl].to(wp)
         _, P, _, mask, gmod = _forward_slice(qq, kk, vv, score_mod, mask_mod, scale, strict, b0,
-                                             want_grad_mod=True)
-        Pd = _rt(P, dtype, strict)
+                                             want_grad_mod=True, _mutant=_mutant)
+        Pd = _rt(P, dtype, strict and _mutant != "p_unrounded")
         dV = torch.matmul(Pd.transpose(-1, -2), dd)
-        dP = _rt(torch.matmul(dd, vv.to(wp).transpose(-1, -2)), dtype, strict)
+        dP = _rt(torch.matmul(dd, vv.to(wp).transpose(-1, -2)), dtype, strict and _mutant != "dp_unrounded")
         delta = (P * dP).sum(dim=-1, keepdim=True)
         dX = P * (dP - delta)
         dS = torch.where(mask, dX * gmod.to(wp), torch.zeros_like(dX)) * scale
-        dS = _rt(dS, dtype, strict)
+        dS = _rt(dS, dtype, strict and _mutant != "ds_unrounded")
         dQ = torch.matmul(dS, kk.to(wp))
         dK = torch.matmul(dS.transpose(-1, -2), qq.to(wp))
         if G > 1:

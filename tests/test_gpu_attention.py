@@ -648,6 +648,26 @@ def test_arbitrary_score_mod_is_linearised(dev, dtype, name, fn):
         att._LINEARISE_BYTES = old
 
 
+PIECEWISE = [
+    ("cap_past_sinks", lambda s, b, h, q, kv: torch.where(kv > 100, torch.tanh(s), s)),
+    ("square_for_late_batches", lambda s, b, h, q, kv: torch.where(b >= 2, 0.2 * s * s, s)),
+    ("sine_for_late_rows", lambda s, b, h, q, kv: torch.where(q >= 64, 3 * torch.sin(s), 2 * s)),
+]
+
+
+@pytest.mark.parametrize("name,fn", PIECEWISE, ids=[a[0] for a in PIECEWISE])
+def test_score_mod_affine_only_near_the_origin(dev, name, fn):
+    """Affine in the score for the first keys / rows / batch entries and something else beyond them: the dense-table
+    lowering must refuse it (it once trusted a corner of the index range) and the call must come out as the reference
+    computes it, which applies the callable to every element (attention.py:59-63)."""
+    from flaxattention_amd.core.common import ScoreModNotLowered, resolve_score_mod
+    print(f"case piecewise score_mod {name}", flush=True)
+    with pytest.raises(ScoreModNotLowered):
+        resolve_score_mod(fn, 2, (3, 2, 200, 333), dev)
+    run(dev, torch.float16, 3, 2, 2, 200, 333, 64, score=fn, oscore=fn, mask=causal_mask, omask=o_causal_mask,
+        strict=False, scale_maxabs=True)
+
+
 def test_lse_is_differentiable(dev):
     """The log-sum-exp output carries a gradient, as in the reference's dense path (attention.py:97-106): a loss of
     sum(O * dO) + sum(lse * w) against torch autograd through a dense fp64 evaluation."""

@@ -94,6 +94,26 @@ def test_score_mod_as_mask(dev):
     check(bm, ref_create_block_mask(o_causal_mask, 1, 2, 256, 256))
 
 
+def test_create_mask_matches_oracle(dev):
+    """The public dense-mask helper (flaxattention/core/blockmask.py:277-322): a tagged mask, an untagged callable that
+    looks at batch and head, a five-argument score_mod (masked where it returns -inf), and B = H = None."""
+    from oracle import ref_create_mask
+
+    def doc(b, h, q_idx, kv_idx):
+        return ((q_idx // 40) == (kv_idx // 40)) & ((h + b) % 2 == 0)
+
+    def as_score(score, b, h, q_idx, kv_idx):
+        return torch.where(q_idx >= kv_idx, score, float("-inf"))
+    for got_fn, want_fn, B, H in ((causal_mask, o_causal_mask, 2, 3), (doc, doc, 2, 3), (as_score, as_score, 1, 2),
+                                  (generate_sliding_window(10), o_sliding_window(10), None, None)):
+        got = fa.create_mask(got_fn, B, H, 100, 130, device=dev)
+        want = ref_create_mask(want_fn, B, H, 100, 130)
+        assert got.dtype == torch.bool and tuple(got.shape) == want.shape
+        assert np.array_equal(got.cpu().numpy(), want)
+    with pytest.raises(ValueError, match="Unknown modification function type"):
+        fa.create_mask(lambda a, b: a, 1, 1, 8, 8, device=dev)
+
+
 def test_sparsity_and_repr(dev):
     bm = fa.create_block_mask(causal_mask, 1, 1, 2048, 2048, device=dev)
     assert abs(bm.sparsity() - 100 * (1 - 136 / 256)) < 1e-9

@@ -126,42 +126,6 @@ def test_decode_matches_prefill_kernel(dev):
     assert max_abs(a.cpu(), b.cpu()) <= 4e-3
 
 
-def test_bench_probes_run(dev):
-    """The bench-only measurement kernels (libflexprobe.so, not part of the product library) launch, report their
-    flop counts and leave finite values behind."""
-    import ctypes
-    import os
-    from flaxattention_amd import _lib
-    L = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libflexprobe.so"))
-    L.flexprobe_last_error.restype = ctypes.c_char_p
-    L.flexprobe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
-    L.flexprobe_mix.argtypes = [ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
-    L.flexprobe_read.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
-    stream = torch.cuda.current_stream(dev).cuda_stream
-    sink = torch.empty(512 * 256, dtype=torch.float32, device=dev)
-    flops = ctypes.c_double(0.0)
-    assert L.flexprobe_mfma(sink.data_ptr(), 4, ctypes.byref(flops), stream) == 0
-    torch.cuda.synchronize()
-    assert flops.value == 512 * 4 * 8 * 4 * 2 * 32 * 32 * 16
-    assert torch.isfinite(sink).all()
-    assert L.flexprobe_mfma(None, 4, None, None) != 0 and b"flexprobe_mfma" in L.flexprobe_last_error()
-    for nm in (8, 12, 16):
-        assert L.flexprobe_mix(sink.data_ptr(), 3, nm, ctypes.byref(flops), stream) == 0
-        torch.cuda.synchronize()
-        assert flops.value == 512 * 4 * nm * 3 * 2 * 32 * 32 * 16
-        assert torch.isfinite(sink).all()
-    assert L.flexprobe_mix(sink.data_ptr(), 3, 7, None, None) != 0 and b"flexprobe_mix" in L.flexprobe_last_error()
-    # the read probe reads its buffer and (practically never) writes the sink
-    src = torch.randint(0, 255, (1 << 20,), dtype=torch.uint8, device=dev)
-    small = torch.zeros(65536, dtype=torch.float32, device=dev)
-    for wgs, nld in ((0, 0), (512, 8), (2048, 1)):
-        assert L.flexprobe_read(src.data_ptr(), src.numel(), small.data_ptr(), wgs, nld, stream) == 0
-    torch.cuda.synchronize()
-    assert float(small.sum()) <= 1.0
-    assert L.flexprobe_read(None, 1 << 20, small.data_ptr(), 0, 0, None) != 0 and b"flexprobe_read" in L.flexprobe_last_error()
-    assert L.flexprobe_read(src.data_ptr(), src.numel(), small.data_ptr(), 0, 3, stream) != 0
-
-
 def test_decode_is_chosen_automatically(dev):
     """Short queries against a long KV cache take the decode kernel without being asked;
     {"decode": False} keeps the forward kernel; both agree, and the gradient path is unaffected."""

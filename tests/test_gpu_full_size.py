@@ -1,6 +1,7 @@
 """The benchmark configurations at their full sizes.  The CPU oracle would need gigabytes of dense
 temporaries there, so the kernels are held to (a) the oracle on a sample of query rows -- a row of O, lse and dQ
-depends on that row of Q and dO and on all of K and V only -- and (b) identities that hold at any size:
+depends on that row of Q and dO and on all of K and V only --, (b) the oracle's dQ, dK and dV on a few whole
+(batch, head) pairs, each a dense problem the host can hold, and (c) identities that hold at any size:
 
     <Q, dQ> = <K, dK>      the loss depends on Q and K through Q K^T only (any score_mod, any mask)
     <V, dV> = <O, dO>      O is linear in V
@@ -66,6 +67,23 @@ def _check_sampled_rows(q, k, v, d_o, out, lse, dq, oscore, omask, dtype, bs, hs
                 assert a <= max(2e-2, ulp) and r <= tol_grad
 
 
+def _check_whole_heads(q, k, v, d_o, dq, dk, dv, oscore, omask, dtype, pairs, tol=1e-3):
+    """dK and dV of key j depend on that key and on ALL of Q and dO (through every row's log-sum-exp and delta), so they
+    are checked on whole (batch, head) pairs: the oracle's backward of one pair is one dense [Lq, Lkv] problem."""
+    for b, h in pairs:
+        s2 = None if oscore is None else (lambda s, bb, hh, qi, ki, h0=h: oscore(s, bb, hh + h0, qi, ki))
+        m2 = None if omask is None else (lambda bb, hh, qi, ki, h0=h: omask(bb, hh + h0, qi, ki))
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        want = ref_attention_bwd(q[sl], k[sl], v[sl], d_o[sl], s2, m2, strict=True)
+        for name, got, w in zip(("dQ", "dK", "dV"), (dq, dk, dv), want):
+            g = got[sl].cpu()
+            a, r = max_abs(g, w), rel_l2(g, w)
+            big = w.abs().max().item()
+            ulp = 2.0 ** (math.floor(math.log2(big)) - (7 if dtype == torch.bfloat16 else 10)) if big > 0 else 0.0
+            print(f"  whole head (b{b},h{h}): {name} max-abs {a:.3e} rel-L2 {r:.3e} (largest entry {big:.1f})", flush=True)
+            assert a <= max(2e-2, ulp) and r <= tol, (name, b, h, a, r)
+
+
 def _inner(a, b):
     return (a.double() * b.double()).sum(dim=(-1, -2))   # per (batch, head)
 
@@ -100,6 +118,7 @@ def test_config2_full_size(dev):
     q, k, v, d_o = _inputs(dev, torch.float16, 8, 8, 2048, 2048, 64)
     out, lse, dq, dk, dv = _fwd_bwd(dev, q, k, v, d_o, generate_checkerboard(2.0, 0.5, "kv"), None)
     _check_sampled_rows(q, k, v, d_o, out, lse, dq, o_checkerboard_kv, None, torch.float16, (0, 7), (0, 5), ROWS)
+    _check_whole_heads(q, k, v, d_o, dq, dk, dv, o_checkerboard_kv, None, torch.float16, ((0, 0), (7, 5)))
     _check_identities(q, k, v, d_o, out.cpu(), dq.cpu(), dk.cpu(), dv.cpu(), additive=False)
     # V = 1: every row of P sums to one
     ones = torch.ones_like(v)
@@ -116,12 +135,13 @@ def test_config3_full_size(dev):
     bm = fa.create_block_mask(causal_mask, 1, 1, 2048, 2048, device=dev)
     out, lse, dq, dk, dv = _fwd_bwd(dev, q, k, v, d_o, generate_alibi_bias(8, -1.0), bm)
     _check_sampled_rows(q, k, v, d_o, out, lse, dq, o_alibi_config(8), o_causal_mask, torch.bfloat16, (0, 7), (0, 7), ROWS)
+    _check_whole_heads(q, k, v, d_o, dq, dk, dv, o_alibi_config(8), o_causal_mask, torch.bfloat16, ((0, 0), (7, 7)))
     _check_identities(q, k, v, d_o, out.cpu(), dq.cpu(), dk.cpu(), dv.cpu(), additive=True)
 
 
 def test_config4_full_size(dev):
-    """bf16 [4,16,8192,128], causal window 1024 + 4 sink keys, tanh soft-cap 50: forward on sampled rows, backward
-    through the identities."""
+    """bf16 [4,16,8192,128], causal window 1024 + 4 sink keys, tanh soft-cap 50: forward and dQ on sampled rows, all
+    three gradients on one whole head, the rest through the identities."""
     print("case config 4 full size", flush=True)
     q, k, v, d_o = _inputs(dev, torch.bfloat16, 4, 16, 8192, 8192, 128)
     bm = fa.create_block_mask(generate_attention_sink(1024, 3), 1, 1, 8192, 8192, device=dev)
@@ -131,6 +151,8 @@ def test_config4_full_size(dev):
     rows = [0, 3, 4, 127, 1023, 1024, 1025, 1028, 4095, 4096, 8191]
     _check_sampled_rows(q, k, v, d_o, out, lse, dq, o_tanh_softcap(50.0), o_sink_window_lt(1024, 4), torch.bfloat16,
                         (0, 3), (0, 15), rows)
+    # one whole head of 8192 x 8192 entries (a few GB of fp32 temporaries on the host)
+    _check_whole_heads(q, k, v, d_o, dq, dk, dv, o_tanh_softcap(50.0), o_sink_window_lt(1024, 4), torch.bfloat16, ((3, 9),))
     _check_identities(q, k, v, d_o, out.cpu(), dq.cpu(), dk.cpu(), dv.cpu(), additive=False)
 
 

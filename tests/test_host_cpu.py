@@ -274,6 +274,39 @@ def test_affine_score_mod_lowering_on_cpu():
     assert affine_score_mod(lambda sc, b, h, q_, k_: sc + 0.0 * q_, 1, 1, 4, 4, "cpu").kind == _lib.SCORE_IDENTITY
 
 
+def test_affine_lowering_checks_the_full_index_range():
+    """A score_mod that is affine in the score near the origin of the index space and something else beyond it
+    must not be lowered to tables (the reference applies the callable to every element,
+    flaxattention/core/attention.py:59-63): the resolver has to refuse it, which hands the call to the
+    linearised path."""
+    import torch
+    from flaxattention_amd.core.common import ScoreModNotLowered, affine_score_mod, resolve_score_mod
+
+    def cap_past_sinks(s, b, h, q, kv):     # identity on the first keys, tanh beyond them
+        return torch.where(kv > 100, torch.tanh(s), s)
+
+    def square_for_late_batches(s, b, h, q, kv):
+        return torch.where(b >= 2, s * s, s)
+
+    def sine_for_late_rows(s, b, h, q, kv):
+        return torch.where(q >= 64, 3 * torch.sin(s), 2 * s)
+
+    cases = [(cap_past_sinks, (1, 2, 256, 256)), (square_for_late_batches, (3, 2, 16, 16)),
+             (sine_for_late_rows, (1, 1, 128, 32))]
+    for fn, shape in cases:
+        assert affine_score_mod(fn, *shape, "cpu") is None, fn.__name__
+        with pytest.raises(ScoreModNotLowered):
+            resolve_score_mod(fn, shape[1], shape, "cpu")
+
+    # the same shapes of callable with an affine far part are still lowered, and the tables carry the far part
+    def scale_past_sinks(s, b, h, q, kv):
+        return torch.where(kv > 100, 0.25 * s - 1.0, s)
+    spec = affine_score_mod(scale_past_sinks, 1, 2, 256, 256, "cpu")
+    assert spec is not None and spec.kind == _lib.SCORE_AFFINE
+    assert float(spec.mul[0, 0, 0, 200]) == 0.25 and float(spec.mul[0, 0, 0, 50]) == 1.0
+    assert float(spec.add[0, 0, 0, 200]) == -1.0 and float(spec.add[0, 0, 0, 50]) == 0.0
+
+
 def test_utils_score_matrix_and_picture(tmp_path):
     """flaxattention/utils.py:17-49, 58-139: dense post-mod scores / mask of one (batch, head) and its picture."""
     from flaxattention_amd.utils import _name_to_title, create_score_mod, visualize_attention_scores

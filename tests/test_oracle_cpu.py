@@ -148,6 +148,50 @@ def test_strict_rounding_points():
     assert max_abs(ref_attention(q32, k32, v32, strict=True), ref_attention(q32, k32, v32, strict=False)) == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16], ids=["f16", "bf16"])
+def test_rounding_points_against_torch_half_program(dtype):
+    """Where the strict oracle rounds through the input dtype is pinned here by a program that torch itself rounds:
+    a literal transcription of flaxattention/core/attention.py:27 (Q.K^T computed in the input dtype, then cast to
+    fp32), :55 (scale applied after the cast), :97-104 (softmax in fp32) and :105 (P cast to the input dtype, then
+    P.V in that dtype) with torch's own 16-bit CPU matrix products, differentiated by torch autograd -- so the
+    backward's rounding of dP = dO.V^T (a product in the input dtype) and of dS (the cotangent of the cast in :27,
+    after the scale) is placed by autograd, not by the oracle's author.  D = 128: the scale is not a power of two, so
+    rounding S before or after it are different numbers.  The oracle must agree with that program to accumulation
+    order, and each misplaced rounding point must not."""
+    from oracle.flex_oracle import MUTANTS
+    q, k, v = seeded_qkv(1, 2, 2, 96, 160, 128, dtype)
+    d_o = torch.randn(1, 2, 96, 128, generator=torch.Generator().manual_seed(5)).to(dtype)
+    scale = 1.0 / math.sqrt(128.0)
+    qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+    S = torch.matmul(qq, kk.transpose(-1, -2)).to(torch.float32) * scale
+    vis = torch.arange(96).view(96, 1) >= torch.arange(160).view(1, 160)
+    S = torch.where(vis, S, torch.full((), -math.inf))
+    P = torch.exp(S - torch.logsumexp(S, dim=-1, keepdim=True))
+    O = torch.matmul(P.to(dtype), vv)
+    O.backward(d_o)
+    literal = (O.detach(), qq.grad, kk.grad, vv.grad)
+
+    def distance(mutant):
+        o = ref_attention(q, k, v, None, o_causal_mask, scale, strict=True, _mutant=mutant)
+        g = ref_attention_bwd(q, k, v, d_o, None, o_causal_mask, scale, strict=True, _mutant=mutant)
+        return [rel_l2(a, b) for a, b in zip((o,) + g, literal)]
+
+    own = distance(None)
+    # measured 3e-5 (fp16) and 0 ... 1e-4 (bf16): accumulation order flips the last bit of a few entries
+    bound = 6e-5 if dtype == torch.float16 else 2e-4
+    assert max(own) <= bound, own
+    touched = {"s_after_scale": (0, 1, 2, 3), "p_unrounded": (0, 3), "dp_unrounded": (1, 2), "ds_unrounded": (1, 2)}
+    for mutant in MUTANTS:
+        d = distance(mutant)
+        for i in touched[mutant]:
+            assert d[i] >= 4 * bound and d[i] >= 4 * own[i], (mutant, i, d, own)
+    # and the variant without round trips is not what that program computes either
+    loose = [rel_l2(a, b) for a, b in zip(
+        (ref_attention(q, k, v, None, o_causal_mask, scale, strict=False),)
+        + ref_attention_bwd(q, k, v, d_o, None, o_causal_mask, scale, strict=False), literal)]
+    assert min(loose) >= 4 * bound, loose
+
+
 # ---- backward ----
 def _autograd(q, k, v, d_o, bias=None, mult=None, keep=None, scale=None):
     qq, kk, vv = (t.double().clone().requires_grad_(True) for t in (q, k, v))
