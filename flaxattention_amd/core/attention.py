@@ -123,13 +123,28 @@ class _Plan:
         # library's default split count, 0 = forward kernel
         self.scale, self.flags, self.decode_splits = float(scale), int(flags), int(decode_splits)
         self.split_kv = True    # the forward kernel may split a call with few query tiles over the keys
+        self.fwd_ws_bytes = None   # bytes of split partials the library wants for the forward (asked on first use)
         self.lists = None       # tile lists for the forward / decode kernels
         self.lists_bwd = None   # tile lists for the backward kernels
         self.keep = [mask.bits, score.mul, score.add]
+        self._params = {}       # parameter blocks by (strides, rows, row offset): a repeated call fills none
 
     def params(self, q, k, v, o, q_index_base: int = 0) -> _lib.FlexAttnParams:
         """q / o may be a slice of rows [q_index_base, q_index_base + q.shape[2]) of the planned query
-        (decode in chunks); everything else refers to the whole problem."""
+        (decode in chunks); everything else refers to the whole problem.  The block is built once per layout and
+        handed out again for the same layout (callers that change a field, as the backward does with d_lse2, copy it)."""
+        key = (q.stride(), k.stride(), v.stride(), o.stride(), q.shape[2], int(q_index_base), id(self.score), id(self.mask),
+               id(self.lists), id(self.lists_bwd))
+        hit = self._params.get(key)
+        if hit is not None:
+            return hit
+        p = self._build_params(q, k, v, o, q_index_base)
+        if len(self._params) > 16:
+            self._params.clear()
+        self._params[key] = p
+        return p
+
+    def _build_params(self, q, k, v, o, q_index_base: int = 0) -> _lib.FlexAttnParams:
         p = _lib.FlexAttnParams()
         p.dtype = _DTYPES[self.dtype]
         p.B, p.Hq, p.Hkv, p.Lq, p.Lkv, p.D, p.Dv = self.B, self.Hq, self.Hkv, q.shape[2], self.Lkv, self.D, self.Dv
@@ -198,6 +213,35 @@ def _make_plan(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, sc
                     plan.lists = lists
                 else:
                     plan.lists_bwd = lists
+    return plan
+
+
+_plans: dict = {}
+
+
+def _plan_for(q, k, v, score_mod, block_mask: Optional[BlockMask], mask_mod, scale, kernel_options) -> _Plan:
+    """_make_plan, remembered for calls that repeat: the same tagged functors (or none), the same BlockMask object,
+    shapes, dtype, scale and options give the same plan, so a training loop lowers nothing and looks nothing up after
+    its first step.  Untagged Python callables are not remembered here: what they capture may change between calls,
+    which their own lowering caches track (common.py)."""
+    def fixed(f, cls):
+        return f is None or f is _identity or (isinstance(f, cls) and getattr(f, "bits", None) is None
+                                               and getattr(f, "kind", 0) != _lib.SCORE_AFFINE)
+    src = block_mask.mask_mod if block_mask is not None else None
+    if not (fixed(score_mod, ScoreMod) and fixed(mask_mod, MaskMod) and fixed(src, MaskMod)):
+        return _make_plan(q, k, v, score_mod, block_mask, mask_mod, scale, kernel_options)
+    try:
+        key = (id(score_mod), id(block_mask), id(mask_mod), tuple(q.shape), tuple(k.shape), tuple(v.shape), q.dtype,
+               q.device, float(scale), tuple(sorted((kernel_options or {}).items())))
+        hit = _plans.get(key)
+    except TypeError:   # an option value that cannot be hashed
+        return _make_plan(q, k, v, score_mod, block_mask, mask_mod, scale, kernel_options)
+    if hit is not None and hit[1] is score_mod and hit[2] is block_mask and hit[3] is mask_mod:
+        return hit[0]
+    plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, scale, kernel_options)
+    if len(_plans) > 64:
+        _plans.clear()
+    _plans[key] = (plan, score_mod, block_mask, mask_mod)   # the objects are held so that their ids stay theirs
     return plan
 
 
@@ -282,11 +326,18 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
                     lse2[:, :, s0:s1] = lc
         else:
             # few query tiles against many keys: with a workspace the library may split the call over the keys
+            # (the library decides from the problem and the device's compute units; 0 = no split.  Asked once per plan)
             ws = None
-            if plan.split_kv and plan.B * plan.Hq * ((plan.Lq + 127) // 128) <= 256 and plan.Lkv >= 1024:
-                nbytes = L.flexattn_fwd_workspace_bytes(p)
-                if nbytes:
-                    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            if plan.split_kv and plan.Lkv >= 1024:
+                if plan.fwd_ws_bytes is None:
+                    # the size also covers the log-sum-exp hand-over of the parity numerics, which this front end
+                    # never needs (it always passes lse2): beyond that part, the bytes are split partials
+                    parity = (plan.flags & _lib.FLAG_PARITY) and not (plan.flags & _lib.FLAG_UNROUNDED)
+                    lse_part = (plan.B * plan.Hq * plan.Lq * 4 + 255) // 256 * 256 if parity else 0
+                    nbytes = int(L.flexattn_fwd_workspace_bytes(p))
+                    plan.fwd_ws_bytes = nbytes if nbytes > lse_part else 0
+                if plan.fwd_ws_bytes:
+                    ws = torch.empty(plan.fwd_ws_bytes, dtype=torch.uint8, device=q.device)
             rc = L.flexattn_fwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(),
                                 ws.data_ptr() if ws is not None else None, _stream(q))
             _lib.check(rc, "flexattn_fwd")
@@ -301,9 +352,15 @@ def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o, d_lse2=None) -> Tuple[Array, Ar
     dq = torch.empty((plan.B, plan.Hq, plan.Lq, plan.D), dtype=q.dtype, device=q.device)
     dk = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.D), dtype=q.dtype, device=q.device)
     dv = torch.empty((plan.B, plan.Hkv, plan.Lkv, plan.Dv), dtype=q.dtype, device=q.device)
-    plan.mask.ensure_transposed()   # the dK/dV kernel reads a bitmap mask packed along the query axis
+    if plan.mask.bits is not None and plan.mask.bits_t is None:
+        plan.mask.ensure_transposed()   # the dK/dV kernel reads a bitmap mask packed along the query axis
+        plan._params.clear()            # parameter blocks made before carry no pointer to the new copy
     p = plan.params(q, k, v, o)
-    p.d_lse2 = d_lse2.data_ptr() if d_lse2 is not None else None
+    if d_lse2 is not None:
+        p2 = _lib.FlexAttnParams()      # a copy: the cached block is shared with other calls
+        _lib.C.memmove(_lib.C.byref(p2), _lib.C.byref(p), _lib.C.sizeof(p))
+        p2.d_lse2 = d_lse2.data_ptr()
+        p = p2
     with torch.cuda.device(q.device):
         ws = torch.empty(max(L.flexattn_bwd_workspace_bytes(p), 256), dtype=torch.uint8, device=q.device)
         rc = L.flexattn_bwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), d_o.data_ptr(),
@@ -544,7 +601,7 @@ def flax_attention(query: Array, key: Array, value: Array, score_mod: Optional[_
         scale = 1.0 / math.sqrt(query.shape[-1])
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     try:
-        plan = _make_plan(q, k, v, score_mod, block_mask, None, scale, kernel_options)
+        plan = _plan_for(q, k, v, score_mod, block_mask, None, scale, kernel_options)
         out, lse2 = _attend(plan, q, k, v)
     except ScoreModNotLowered:
         out, lse2 = _attend_linearised(q, k, v, score_mod, block_mask, None, scale, kernel_options)
@@ -630,7 +687,7 @@ def flax_attention_pallas(query: Array, key: Array, value: Array, score_mod: Opt
         return out if bhln else out.transpose(1, 2)
     q, k, v = map(_as_kernel_layout, _pad_head_dims(query, key, value, kernel_options))
     try:
-        plan = _make_plan(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
+        plan = _plan_for(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
         out, _ = _attend(plan, q, k, v)
     except ScoreModNotLowered:
         out, _ = _attend_linearised(q, k, v, score_mod, block_mask, mask_mod, sm_scale, kernel_options)
