@@ -393,19 +393,20 @@ class _FlexAttention(torch.autograd.Function):
 _LINEARISE_BYTES = 2 << 30   # dense fp32 temporaries of one batch chunk (scores, mod, derivative, the two tables)
 
 
-def _linearised_tables(score_fn, q, k, scale: float, b0: int):
+def _linearised_tables(score_fn, q, k, scale: float, b0: int, h0: int = 0):
     """For an arbitrary differentiable scalar score_mod f: the scaled scores S0 of the call (the product computed in
     the input dtype and cast to fp32, then scaled: attention.py:27, 55), Y = f(S0, b, h, q_idx, kv_idx) and
     G = dY/dS0, as the dense fp32 tables of the affine functor  mul * s + add  with mul = G and add = Y - G * S0.
     At s = S0 that is f(S0) exactly, its derivative is f'(S0), and where a kernel's own score differs from S0 in the
-    last bit of the input dtype the difference enters to first order.  `b0` is the batch index of q[0]."""
+    last bit of the input dtype the difference enters to first order.  `b0` / `h0` are the batch and head index of
+    q[0, 0] in the whole problem."""
     B, Hq, Lq, _ = q.shape
     G_ = Hq // k.shape[1]
     kk = k if G_ == 1 else k.repeat_interleave(G_, dim=1)   # the reference repeats K for GQA (attention.py:80-82)
     s0 = (torch.matmul(q, kk.transpose(-1, -2)).to(torch.float32) * scale).requires_grad_(True)
     dev = q.device
     b = torch.arange(b0, b0 + B, dtype=torch.int32, device=dev).reshape(B, 1, 1, 1)
-    h = torch.arange(Hq, dtype=torch.int32, device=dev).reshape(1, Hq, 1, 1)
+    h = torch.arange(h0, h0 + Hq, dtype=torch.int32, device=dev).reshape(1, Hq, 1, 1)
     qi = torch.arange(Lq, dtype=torch.int32, device=dev).reshape(1, 1, Lq, 1)
     ki = torch.arange(k.shape[2], dtype=torch.int32, device=dev).reshape(1, 1, 1, -1)
     with torch.enable_grad():
@@ -420,44 +421,55 @@ def _linearised_tables(score_fn, q, k, scale: float, b0: int):
     return g.contiguous(), add.contiguous()
 
 
+def _linearise_chunks(B: int, Hq: int, Hkv: int, Lq: int, Lkv: int):
+    """(b0, b1, h0, h1) slabs of the problem whose dense fp32 temporaries (scores, mod, derivative and the two
+    tables: five [Lq, Lkv] planes per head) stay within _LINEARISE_BYTES: whole batch elements while one fits, else
+    whole groups of query heads that share a KV head (one group at least: a single head of 8192 x 8192 is 1.3 GB)."""
+    per_head = 5 * Lq * Lkv * 4
+    G = Hq // Hkv
+    if per_head * Hq <= _LINEARISE_BYTES:
+        step = max(1, min(B, _LINEARISE_BYTES // max(per_head * Hq, 1)))
+        return [(b0, min(b0 + step, B), 0, Hq) for b0 in range(0, B, step)]
+    heads = max(G, (_LINEARISE_BYTES // max(per_head, 1)) // G * G)
+    return [(b, b + 1, h0, min(h0 + heads, Hq)) for b in range(B) for h0 in range(0, Hq, heads)]
+
+
 class _FlexAttentionLinearised(torch.autograd.Function):
     """flax_attention for a score_mod outside the functor families and not affine in the score (the reference applies
-    any scalar callable, attention.py:59-63).  Per chunk of batch elements the callable and its derivative are
-    evaluated at the call's own scores and handed to the kernels as the tables of an affine functor; the backward
-    evaluates them again instead of keeping them."""
+    any scalar callable, attention.py:59-63).  Per slab of batch elements (or, when one batch element is too large,
+    of query-head groups) the callable and its derivative are evaluated at the call's own scores and handed to the
+    kernels as the tables of an affine functor; the backward evaluates them again instead of keeping them."""
 
     @staticmethod
     def forward(ctx, q, k, v, cfg):
-        score_fn, block_mask, mask_mod, scale, opts = cfg
         B, Hq, Lq, _ = q.shape
-        per_b = 5 * Hq * Lq * k.shape[2] * 4
-        step = max(1, min(B, _LINEARISE_BYTES // max(per_b, 1)))
+        G = Hq // k.shape[1]
         o = torch.empty((B, Hq, Lq, v.shape[3]), dtype=q.dtype, device=q.device)
         lse2 = torch.empty((B, Hq, Lq), dtype=torch.float32, device=q.device)
-        chunks = []
-        for b0 in range(0, B, step):
-            b1 = min(b0 + step, B)
-            plan = _FlexAttentionLinearised._chunk_plan(cfg, q[b0:b1], k[b0:b1], v[b0:b1], b0)
-            oc, lc = _run_fwd(plan, q[b0:b1], k[b0:b1], v[b0:b1])
-            o[b0:b1], lse2[b0:b1] = oc, lc
+        chunks = _linearise_chunks(B, Hq, k.shape[1], Lq, k.shape[2])
+        for b0, b1, h0, h1 in chunks:
+            qc, kc, vc = q[b0:b1, h0:h1], k[b0:b1, h0 // G:h1 // G], v[b0:b1, h0 // G:h1 // G]
+            plan = _FlexAttentionLinearised._chunk_plan(cfg, qc, kc, vc, b0, h0)
+            oc, lc = _run_fwd(plan, qc, kc, vc)
+            o[b0:b1, h0:h1], lse2[b0:b1, h0:h1] = oc, lc
             plan.score = None   # the tables are not kept for the backward
-            chunks.append((b0, b1))
         ctx.save_for_backward(q, k, v, o, lse2)
         ctx.cfg, ctx.chunks = cfg, chunks
         ctx.set_materialize_grads(False)
         return o, lse2
 
     @staticmethod
-    def _chunk_plan(cfg, qc, kc, vc, b0):
+    def _chunk_plan(cfg, qc, kc, vc, b0, h0=0):
         score_fn, block_mask, mask_mod, scale, opts = cfg
-        mul, add = _linearised_tables(score_fn, qc, kc, scale, b0)
+        mul, add = _linearised_tables(score_fn, qc, kc, scale, b0, h0)
         score = ScoreMod(_lib.SCORE_AFFINE, name=getattr(score_fn, "__name__", "score_mod"), mul=mul, add=add, fn=score_fn)
-        # the mask of this chunk: a functor that does not look at the batch index serves as it is; anything else is the
-        # user's callable with the chunk's batch offset (lowered again for the chunk)
+        # the mask of this slab: a functor that does not look at the batch (or head) index serves as it is; anything
+        # else is the user's callable with the slab's offsets (lowered again for the slab; the lowering is remembered
+        # by the callable's code and offsets, so the backward finds the forward's)
         src = block_mask.mask_mod if block_mask is not None else mask_mod
         spec = block_mask.spec if block_mask is not None else (src if isinstance(src, MaskMod) else None)
-        if not (isinstance(spec, MaskMod) and (spec.bits is None or spec.bits.shape[0] == 1)):
-            spec = None if src is None else (lambda b, h, q_idx, kv_idx: src(b + b0, h, q_idx, kv_idx))
+        if not (isinstance(spec, MaskMod) and (spec.bits is None or (spec.bits.shape[0] == 1 and (h0 == 0 or spec.bits.shape[1] == 1)))):
+            spec = None if src is None else (lambda b, h, q_idx, kv_idx: src(b + b0, h + h0, q_idx, kv_idx))
         plan = _make_plan(qc, kc, vc, IDENTITY, None, spec, scale, opts)
         plan.score = score
         plan.keep = [plan.mask.bits, mul, add]
@@ -468,12 +480,14 @@ class _FlexAttentionLinearised(torch.autograd.Function):
         q, k, v, o, lse2 = ctx.saved_tensors
         if d_o is None:
             d_o = torch.zeros_like(o)
+        G = q.shape[1] // k.shape[1]
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-        for b0, b1 in ctx.chunks:
-            plan = _FlexAttentionLinearised._chunk_plan(ctx.cfg, q[b0:b1], k[b0:b1], v[b0:b1], b0)
-            dl = None if d_lse2 is None else d_lse2[b0:b1]
-            dq[b0:b1], dk[b0:b1], dv[b0:b1] = _run_bwd(plan, q[b0:b1], k[b0:b1], v[b0:b1], o[b0:b1], lse2[b0:b1],
-                                                        d_o[b0:b1], dl)
+        for b0, b1, h0, h1 in ctx.chunks:
+            qc, kc, vc = q[b0:b1, h0:h1], k[b0:b1, h0 // G:h1 // G], v[b0:b1, h0 // G:h1 // G]
+            plan = _FlexAttentionLinearised._chunk_plan(ctx.cfg, qc, kc, vc, b0, h0)
+            dl = None if d_lse2 is None else d_lse2[b0:b1, h0:h1]
+            dq[b0:b1, h0:h1], dk[b0:b1, h0 // G:h1 // G], dv[b0:b1, h0 // G:h1 // G] = _run_bwd(
+                plan, qc, kc, vc, o[b0:b1, h0:h1], lse2[b0:b1, h0:h1].contiguous(), d_o[b0:b1, h0:h1], dl)
         return dq, dk, dv, None
 
 

@@ -317,9 +317,10 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
     # a lowering is cached only together with what it was derived from: the callable and the captured tensors
     # at their current versions (a learned bias that the optimizer has updated in place must be read again)
     stamp = _capture_stamp(fn)
-    key = (id(fn), H, None if shape is None else tuple(shape), str(device))   # a family is verified per problem shape
+    who = _callable_key(fn, stamp)
+    key = (who, H, None if shape is None else tuple(shape), str(device))   # a family is verified per problem shape
     hit = _score_cache.get(key)
-    if hit is not None and not (hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp)):
+    if hit is not None and not (_same_callable(hit[0], fn) and stamp is not None and _stamp_valid(hit[2], stamp)):
         hit = None
     if hit is not None and hit[1] is not None:
         return hit[1]
@@ -332,9 +333,9 @@ def resolve_score_mod(fn: Optional[Callable], H: int, shape: Optional[Tuple[int,
         if spec is not None:
             return spec
     if shape is not None and device is not None:
-        key = ("affine", id(fn)) + tuple(shape) + (str(device),)
+        key = ("affine", who) + tuple(shape) + (str(device),)
         hit = _score_cache.get(key)
-        if hit is not None and hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp):
+        if hit is not None and _same_callable(hit[0], fn) and stamp is not None and _stamp_valid(hit[2], stamp):
             return hit[1]
         spec = affine_score_mod(fn, *shape, device)
         if spec is not None:
@@ -558,6 +559,31 @@ def _capture_stamp(fn):
     return [(t, t._version) for t in tensors] + [(None, tuple(scalars))]
 
 
+def _callable_key(fn, stamp):
+    """Cache key of a callable.  A plain function or lambda whose captures can all be seen is known by its code object
+    and by what it captures (numbers and strings by value, tensors by identity), so that a closure made anew for every
+    call -- `lambda s, b, h, q, kv: s + bias[h]` inside a training step -- finds the lowering of its predecessor;
+    anything else (a partial, a bound method, a callable with hidden state) is known by its identity."""
+    code = getattr(fn, "__code__", None)
+    if code is None or stamp is None:
+        return ("id", id(fn))
+    try:
+        key = ("code", code, stamp[-1][1], tuple(id(t) for t, _ in stamp[:-1]))
+        hash(key)
+        return key
+    except TypeError:
+        return ("id", id(fn))
+
+
+def _same_callable(cached, fn) -> bool:
+    """`fn` is the callable a cache entry was made from, or another instance of the same code (what it captures is
+    compared by the caller through the stamps)."""
+    if cached is fn:
+        return True
+    code = getattr(fn, "__code__", None)
+    return code is not None and getattr(cached, "__code__", None) is code
+
+
 def _stamp_valid(stamp, now=None) -> bool:
     """`stamp` (taken when a lowering was cached) still describes the callable: the same tensors at the same
     versions.  `now` is a fresh stamp of the callable (a closure variable may have been rebound to another tensor)."""
@@ -710,9 +736,9 @@ def resolve_mask_mod(fn: Optional[Callable], B: int, H: int, Q: int, KV: int, de
     Qp, KVp = _pad128(Q), _pad128(KV)
     # the dense evaluation is remembered per callable, shape and the captured tensors at their versions
     stamp = _capture_stamp(fn)
-    key = (id(fn), B, H, Q, KV, str(device), real)
+    key = (_callable_key(fn, stamp), B, H, Q, KV, str(device), real)
     hit = _mask_cache.get(key)
-    if hit is not None and hit[0] is fn and stamp is not None and _stamp_valid(hit[2], stamp):
+    if hit is not None and _same_callable(hit[0], fn) and stamp is not None and _stamp_valid(hit[2], stamp):
         return hit[1]
     spec = _lower_mask_callable(fn, B, H, Q, KV, Qp, KVp, device, real)
     if stamp is not None:

@@ -648,6 +648,23 @@ def test_arbitrary_score_mod_is_linearised(dev, dtype, name, fn):
         att._LINEARISE_BYTES = old
 
 
+def test_linearised_score_mod_in_head_group_slabs(dev):
+    """When the dense temporaries of ONE batch element exceed the budget, the linearised path walks groups of query
+    heads that share a KV head; the callable and a head-dependent mask must still see absolute batch and head indices."""
+    import flaxattention_amd.core.attention as att
+    print("case linearised score_mod, head-group slabs", flush=True)
+    fn = lambda s, b, h, q, kv: torch.where(s > 0, s, 0.25 * (h + 1) * s) * (1.0 + 0.5 * b)   # noqa: E731
+    by_head = lambda b, h, q, kv: (q >= kv) | ((h % 2 == 1) & (kv < 8))                            # noqa: E731
+    old = att._LINEARISE_BYTES
+    att._LINEARISE_BYTES = 5 * 2 * 200 * 333 * 4   # two heads = one group of the 4 query / 2 KV heads
+    try:
+        assert att._linearise_chunks(2, 4, 2, 200, 333) == [(0, 1, 0, 2), (0, 1, 2, 4), (1, 2, 0, 2), (1, 2, 2, 4)]
+        run(dev, torch.float16, 2, 4, 2, 200, 333, 64, score=fn, oscore=fn, mask=by_head, omask=by_head, strict=False,
+            scale_maxabs=True)
+    finally:
+        att._LINEARISE_BYTES = old
+
+
 PIECEWISE = [
     ("cap_past_sinks", lambda s, b, h, q, kv: torch.where(kv > 100, torch.tanh(s), s)),
     ("square_for_late_batches", lambda s, b, h, q, kv: torch.where(b >= 2, 0.2 * s * s, s)),

@@ -307,6 +307,43 @@ def test_affine_lowering_checks_the_full_index_range():
     assert float(spec.add[0, 0, 0, 200]) == -1.0 and float(spec.add[0, 0, 0, 50]) == 0.0
 
 
+def test_lowering_cache_serves_closures_made_anew():
+    """A score_mod written as a lambda inside the training step is a new function object on every call; its lowering
+    is found again through its code object and what it captures (numbers by value, tensors by identity and version),
+    and is made anew when any of that changes."""
+    import torch
+    from flaxattention_amd.core import common
+    calls = []
+    orig = common._probe_score_mod
+
+    def counting(*a, **k):
+        calls.append(1)
+        return orig(*a, **k)
+    common._probe_score_mod = counting
+    try:
+        def make(f):
+            return lambda s, b, h, q, kv: torch.where((kv - q) % 2 == 0, s * f, s * 0.5)
+        shape = (1, 4, 64, 64)
+        a = common.resolve_score_mod(make(2.0), 4, shape, "cpu")
+        b = common.resolve_score_mod(make(2.0), 4, shape, "cpu")
+        assert a is b and len(calls) == 1 and a.kind == _lib.SCORE_CHECKERBOARD and a.p0 == 2.0
+        c = common.resolve_score_mod(make(3.0), 4, shape, "cpu")          # another captured number: another lowering
+        assert c is not a and c.p0 == 3.0 and len(calls) == 2
+        assert common.resolve_score_mod(make(2.0), 4, shape, "cpu") is a  # both stay cached side by side
+        bias = torch.zeros(4)
+
+        def with_table():
+            return lambda s, b, h, q, kv: s + bias[h.long()]
+        t1 = common.resolve_score_mod(with_table(), 4, shape, "cpu")
+        n = len(calls)
+        assert common.resolve_score_mod(with_table(), 4, shape, "cpu") is t1 and len(calls) == n
+        bias.add_(1.0)                                                    # in-place update: read again
+        t2 = common.resolve_score_mod(with_table(), 4, shape, "cpu")
+        assert t2 is not t1 and float(t2.add.reshape(-1)[0]) == 1.0
+    finally:
+        common._probe_score_mod = orig
+
+
 def test_utils_score_matrix_and_picture(tmp_path):
     """flaxattention/utils.py:17-49, 58-139: dense post-mod scores / mask of one (batch, head) and its picture."""
     from flaxattention_amd.utils import _name_to_title, create_score_mod, visualize_attention_scores
