@@ -33,6 +33,12 @@ Parity pinning status (what checks each function independently of this file):
   brute-force loop on tiny inputs, and algebraic invariants.
 * ref_attention_bwd: pinned by torch autograd through an fp64 dense forward
   and by finite differences.
+* strict=True, placement of the 16-bit rounding points (S before the scale, P,
+  dP, dS after the scale): pinned by a literal transcription of
+  attention.py:27, 55, 97-105 with torch's own fp16 / bf16 CPU matrix products,
+  differentiated by torch autograd (so autograd, not this file's author, places
+  the backward's roundings), and by four deliberately misplaced roundings
+  (MUTANTS below) that the test must tell apart from the real thing.
 * PARITY UNPINNED: whether the reference's XLA executable really performs the
   input-dtype round trips on S, P, dP and dS (``strict=True``) or elides them
   (``strict=False``).  Both variants are provided; no fixture can decide.
