@@ -291,7 +291,30 @@ def _holder_for(mask: MaskMod) -> BlockMask:
 
 
 def _stream(t) -> int:
+    """Raw handle of torch's current stream on the tensor's device (the private accessor skips the Stream object
+    that torch.cuda.current_stream builds on every call)."""
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        return raw(t.device.index if t.device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+class _on_device:
+    """torch.cuda.device(dev) only when dev is not already current (entering the context costs ~10 us of host time)."""
+    __slots__ = ("ctx",)
+
+    def __init__(self, dev):
+        idx = dev.index
+        self.ctx = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
 
 
 def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
@@ -299,7 +322,7 @@ def _run_fwd(plan: _Plan, q, k, v) -> Tuple[Array, Array]:
     o = torch.empty((plan.B, plan.Hq, plan.Lq, plan.Dv), dtype=q.dtype, device=q.device)
     lse2 = torch.empty((plan.B, plan.Hq, plan.Lq), dtype=torch.float32, device=q.device)
     p = plan.params(q, k, v, o)
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         if plan.decode_splits != 0:
             splits = max(plan.decode_splits, 0)   # 0 asks the library for its default
             rows = max(_decode_columns(plan.D) // (plan.Hq // plan.Hkv), 1)   # query rows one decode call takes
@@ -361,7 +384,7 @@ def _run_bwd(plan: _Plan, q, k, v, o, lse2, d_o, d_lse2=None) -> Tuple[Array, Ar
         _lib.C.memmove(_lib.C.byref(p2), _lib.C.byref(p), _lib.C.sizeof(p))
         p2.d_lse2 = d_lse2.data_ptr()
         p = p2
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         ws = torch.empty(max(L.flexattn_bwd_workspace_bytes(p), 256), dtype=torch.uint8, device=q.device)
         rc = L.flexattn_bwd(p, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), lse2.data_ptr(), d_o.data_ptr(),
                             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), _stream(q))
