@@ -46,13 +46,34 @@ PEAK_HBM_GBPS = 8000.0
 # HBM bytes per launch.  A timing run cannot read hardware counters, so these are copied from the counter runs
 # summarised in TRAFFIC_SOURCE (two `rocprofv3 --pmc` runs of `python3 bench.py --pmc-probe`, FETCH_SIZE then
 # WRITE_SIZE, each scaled by what the same counter reads for the 1 GiB device copy at the start of that run).
-# Keyed by (workload, kernel); a kernel that has not been measured reports null.
+# Keyed by (workload, kernel); a kernel that has not been measured reports null -- and so does every kernel once the
+# kernel sources differ from the ones the counters were read for (TRAFFIC_KERNEL_SHA), so that a copied figure
+# cannot outlive the code it describes.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_config2_and_decode_pmc.md"
+TRAFFIC_KERNEL_FILES = ("fwd_mfma.cuh", "bwd_mfma.cuh", "mfma_common.cuh")
+TRAFFIC_KERNEL_SHA = "1417a4fd402899bf"
 MEASURED_TRAFFIC_BYTES = {
-    ("config2", "fwd_pipe_kernel"): 67954311,
-    ("config2", "bwd_dq_kernel"): 136180161,
-    ("config2", "bwd_dkv_kernel"): 137453189,
+    ("config2", "fwd_pipe_kernel"): 67971461,
+    ("config2", "bwd_dq_kernel"): 135903766,
+    ("config2", "bwd_dkv_kernel"): 137505327,
 }
+
+
+def kernel_sources_sha():
+    import hashlib
+    h = hashlib.sha256()
+    for f in TRAFFIC_KERNEL_FILES:
+        h.update(open(os.path.join(ROOT, "flaxattention_amd", "csrc", f), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel):
+    try:
+        if kernel_sources_sha() != TRAFFIC_KERNEL_SHA:
+            return None
+    except OSError:
+        return None
+    return MEASURED_TRAFFIC_BYTES.get((workload, kernel))
 
 
 def log(*a):
@@ -495,7 +516,7 @@ def main():
         "kernels": r["kernels"],
         "roofline": {"bound": "mfma", "kernel": dom, "achieved": kd["tflops"], "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(kd["tflops"] / PEAK_MFMA_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, dom)), "traffic_source": TRAFFIC_SOURCE,
+                     "traffic": measured_traffic(a.workload, dom), "traffic_source": TRAFFIC_SOURCE,
                      "duration_source": "HIP events around the kernel inside the step (average over the steps); rocprofv3 --kernel-trace of "
                                         "this command agrees (profiles/fwd_bwd_config2_kernel_trace.md)",
                      "attribution": "S and dP are computed by both backward kernels; they are attributed to bwd_dkv_kernel "
