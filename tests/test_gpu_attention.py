@@ -685,6 +685,56 @@ def test_score_mod_affine_only_near_the_origin(dev, name, fn):
         strict=False, scale_maxabs=True)
 
 
+def test_repeated_calls_reuse_the_plan_and_stay_correct(dev):
+    """A training loop calls the front end with the same functors, block mask, shapes and options: the plan (lowered
+    functors, tile lists, parameter block) is made once and found again.  A different block mask, other shapes, other
+    options or another layout of the same shapes must not be served the remembered one."""
+    import flaxattention_amd.core.attention as att
+    made = []
+    orig = att._make_plan
+
+    def counting(*a, **k):
+        made.append(1)
+        return orig(*a, **k)
+    att._make_plan = counting
+    try:
+        q, k, v = (t.to(dev) for t in seeded_qkv(2, 4, 4, 256, 256, 64, torch.float16))
+        score = generate_alibi_bias(4, -1.0)
+        bm = fa.create_block_mask(causal_mask, 1, 1, 256, 256, device=dev)
+        want = ref_attention(q.cpu(), k.cpu(), v.cpu(), o_alibi_config(4), o_causal_mask)
+        a = fa.flax_attention(q, k, v, score_mod=score, block_mask=bm)
+        n = len(made)
+        b = fa.flax_attention(q, k, v, score_mod=score, block_mask=bm)
+        assert len(made) == n and torch.equal(a, b)
+        close(a, want, torch.float16, "O, remembered plan")
+        # [B,L,H,D] storage of the same logical shapes: same plan, another parameter block (strides)
+        qt, kt, vt = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v))
+        c = fa.flax_attention(qt, kt, vt, score_mod=score, block_mask=bm)
+        assert len(made) == n and torch.equal(a, c)
+        # another mask object, other options, other shapes: planned anew, and right
+        window = fa.create_block_mask(generate_sliding_window(40), 1, 1, 256, 256, device=dev)
+        d = fa.flax_attention(q, k, v, score_mod=score, block_mask=window)
+        assert len(made) == n + 1
+        close(d, ref_attention(q.cpu(), k.cpu(), v.cpu(), o_alibi_config(4), o_sliding_window(40)), torch.float16, "O, other mask")
+        e = fa.flax_attention(q, k, v, score_mod=score, block_mask=bm, kernel_options={"numerics": "parity"})
+        assert len(made) == n + 2
+        close(e, want, torch.float16, "O, other options")
+        f = fa.flax_attention(q[:, :, :128], k, v, score_mod=score, block_mask=bm)
+        assert len(made) == n + 3
+        close(f, want[:, :, :128], torch.float16, "O, fewer rows")
+        # gradients through a remembered plan, twice in a row
+        for _ in range(2):
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            fa.flax_attention(qq, kk, vv, score_mod=score, block_mask=bm).sum().backward()
+            wq, wk, wv = ref_attention_bwd(q.cpu(), k.cpu(), v.cpu(), torch.ones_like(want), o_alibi_config(4), o_causal_mask)
+            close(qq.grad, wq, torch.float16, "dQ, remembered plan", scale_maxabs=True)
+            close(kk.grad, wk, torch.float16, "dK, remembered plan", scale_maxabs=True)
+            close(vv.grad, wv, torch.float16, "dV, remembered plan", scale_maxabs=True)
+        assert len(made) == n + 3
+    finally:
+        att._make_plan = orig
+
+
 def test_lse_is_differentiable(dev):
     """The log-sum-exp output carries a gradient, as in the reference's dense path (attention.py:97-106): a loss of
     sum(O * dO) + sum(lse * w) against torch autograd through a dense fp64 evaluation."""
