@@ -426,6 +426,25 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
 
 
+def test_bench_traffic_figures_do_not_outlive_the_kernels():
+    """The HBM-traffic figures in bench.py are copied from hardware-counter runs; they are reported only while the
+    kernel sources are the ones they were measured for (a hash), and read null after any change to them."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.kernel_sources_sha() == bench.TRAFFIC_KERNEL_SHA, \
+        "kernel sources changed: re-run the counter passes named in profiles/hbm_traffic_config2_and_decode_pmc.md"
+    assert bench.measured_traffic("config2", "bwd_dkv_kernel") == bench.MEASURED_TRAFFIC_BYTES[("config2", "bwd_dkv_kernel")]
+    assert bench.measured_traffic("config2", "no_such_kernel") is None
+    old = bench.TRAFFIC_KERNEL_SHA
+    bench.TRAFFIC_KERNEL_SHA = "0" * 16
+    try:
+        assert bench.measured_traffic("config2", "bwd_dkv_kernel") is None
+    finally:
+        bench.TRAFFIC_KERNEL_SHA = old
+
+
 def test_block_classes_of_a_bitmap():
     """The table the fused kernels consult inside partial tiles: 1 = block entirely visible, 2 = entirely hidden."""
     from flaxattention_amd.core.common import block_classes
